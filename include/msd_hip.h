@@ -1,0 +1,154 @@
+/*
+ * C ABI of libmsd_hip.so: dilated 3x3 (2D) / 3x3x3 (3D) convolution with
+ * symmetric ("reflection") padding, optional fused ReLU, forward and backward,
+ * on AMD gfx950 (MI355X).
+ *
+ * One entry point per operator that the reference exports from its pybind11
+ * module `msd_custom_convolutions` (msd_custom_convolutions.cpp:343-369); the
+ * 2D/3D and float/double variants that the reference selects by tensor rank
+ * and AT_DISPATCH_FLOATING_TYPES (torch_cuda_dispatch.cu:95-441) are selected
+ * here by the `ndim` and `dtype` arguments.
+ *
+ * Conventions
+ *   - every data pointer is DEVICE memory on the current HIP device;
+ *   - a tensor view is a base pointer plus `ndim + 2` ELEMENT strides in the
+ *     order {batch, channel, [z,] y, x}; views may be channel slices of a larger
+ *     allocation (the dense block's growing stack, msd_block.py:30-46).
+ *     Strides must be non-negative and no two elements of an output view may alias;
+ *   - `spatial` holds `ndim` extents, {H, W} or {D, H, W};
+ *   - weights are contiguous (c_out, c_in, 3, 3[, 3]); bias is contiguous (c_out);
+ *   - 0 < dilation <= every spatial extent (msd_custom_convolutions.cpp:39-52),
+ *     so a single fold of the index suffices;
+ *   - `stream` is a hipStream_t (NULL = the default stream); calls are
+ *     asynchronous and never synchronise the host;
+ *   - return value 0 = success; otherwise an MSD_ERR_* code, and
+ *     msd_last_error() returns a message for the calling thread.
+ *   - the caller owns every buffer; `output` is overwritten; `grad_input`,
+ *     `grad_kernel` and `grad_bias` are ACCUMULATED into
+ *     (conv2d_backward_x.cu:103,205; conv2d_backward_k.cu:52,105;
+ *     conv2d_backward_bias.cu:46).
+ *   - results are deterministic: weight and bias gradients are reduced in a
+ *     fixed order through `workspace` (the reference uses float atomics).
+ */
+#ifndef MSD_HIP_H
+#define MSD_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MSD_F32 0
+#define MSD_F64 1
+
+#define MSD_OK 0
+#define MSD_ERR_INVALID 1   /* bad argument; nothing was launched */
+#define MSD_ERR_HIP 2       /* the HIP runtime reported an error */
+#define MSD_ERR_WORKSPACE 3 /* workspace missing or too small */
+
+/* Message describing the last failure on the calling thread ("" if none). */
+const char *msd_last_error(void);
+
+/* ABI version of this header: bumped on any incompatible change. */
+int msd_abi_version(void);
+
+/*
+ * Bytes of device scratch that msd_conv_backward_k, msd_conv_relu_backward_k,
+ * msd_conv_relu_backward_kb and msd_conv_relu_backward_bias need for this
+ * problem (partial sums of the fixed-order reduction).  Returns < 0 on
+ * invalid arguments.
+ */
+int64_t msd_workspace_bytes(int dtype, int ndim, int64_t batch, int64_t c_in, int64_t c_out,
+                            const int64_t *spatial);
+
+/* y = bias + conv(x).  Replaces conv_forward, msd_custom_convolutions.cpp:85-117
+ * (kernels conv2d_forward.cu:22-93, conv3d_forward.cu:22-108). */
+int msd_conv_forward(int dtype, int ndim, int64_t batch, int64_t c_in, int64_t c_out,
+                     const int64_t *spatial, int dilation,
+                     const void *input, const int64_t *input_strides,
+                     const void *kernel, const void *bias,
+                     void *output, const int64_t *output_strides, void *stream);
+
+/* y = max(0, bias + conv(x)).  Replaces conv_relu_forward,
+ * msd_custom_convolutions.cpp:213-245 (kernels conv2d_forward.cu:95-174,
+ * conv3d_forward.cu:110-196). */
+int msd_conv_relu_forward(int dtype, int ndim, int64_t batch, int64_t c_in, int64_t c_out,
+                          const int64_t *spatial, int dilation,
+                          const void *input, const int64_t *input_strides,
+                          const void *kernel, const void *bias,
+                          void *output, const int64_t *output_strides, void *stream);
+
+/* grad_input += conv^T(grad_output).  Replaces conv_backward_x,
+ * msd_custom_convolutions.cpp:119-148 (kernels conv2d_backward_x.cu:13-106,
+ * conv3d_backward_x.cu:13-123). */
+int msd_conv_backward_x(int dtype, int ndim, int64_t batch, int64_t c_in, int64_t c_out,
+                        const int64_t *spatial, int dilation,
+                        const void *grad_output, const int64_t *grad_output_strides,
+                        const void *kernel,
+                        void *grad_input, const int64_t *grad_input_strides, void *stream);
+
+/* grad_input += conv^T(grad_output * [0 < output]).  Replaces conv_relu_backward_x,
+ * msd_custom_convolutions.cpp:247-281 (kernels conv2d_backward_x.cu:109-208,
+ * conv3d_backward_x.cu:125-241). */
+int msd_conv_relu_backward_x(int dtype, int ndim, int64_t batch, int64_t c_in, int64_t c_out,
+                             const int64_t *spatial, int dilation,
+                             const void *output, const int64_t *output_strides,
+                             const void *grad_output, const int64_t *grad_output_strides,
+                             const void *kernel,
+                             void *grad_input, const int64_t *grad_input_strides, void *stream);
+
+/* grad_kernel += d/dk.  Replaces conv_backward_k, msd_custom_convolutions.cpp:150-178
+ * (kernels conv2d_backward_k.cu:12-59, conv3d_backward_k.cu:11-64). */
+int msd_conv_backward_k(int dtype, int ndim, int64_t batch, int64_t c_in, int64_t c_out,
+                        const int64_t *spatial, int dilation,
+                        const void *grad_output, const int64_t *grad_output_strides,
+                        const void *input, const int64_t *input_strides,
+                        void *grad_kernel,
+                        void *workspace, int64_t workspace_bytes, void *stream);
+
+/* grad_kernel += d/dk with the ReLU mask.  Replaces conv_relu_backward_k,
+ * msd_custom_convolutions.cpp:283-316 (kernels conv2d_backward_k.cu:61-112,
+ * conv3d_backward_k.cu:66-122). */
+int msd_conv_relu_backward_k(int dtype, int ndim, int64_t batch, int64_t c_in, int64_t c_out,
+                             const int64_t *spatial, int dilation,
+                             const void *output, const int64_t *output_strides,
+                             const void *grad_output, const int64_t *grad_output_strides,
+                             const void *input, const int64_t *input_strides,
+                             void *grad_kernel,
+                             void *workspace, int64_t workspace_bytes, void *stream);
+
+/* grad_bias += sum over batch and voxels of grad_output.  Replaces conv_backward_bias,
+ * msd_custom_convolutions.cpp:180-211 (a torch sum in the reference). */
+int msd_conv_backward_bias(int dtype, int ndim, int64_t batch, int64_t c_out,
+                           const int64_t *spatial,
+                           const void *grad_output, const int64_t *grad_output_strides,
+                           void *grad_bias,
+                           void *workspace, int64_t workspace_bytes, void *stream);
+
+/* grad_bias += sum of grad_output where 0 < output.  Replaces conv_relu_backward_bias,
+ * msd_custom_convolutions.cpp:318-338 (kernels conv2d_backward_bias.cu:12-49,
+ * conv3d_backward_bias.cu:12-51). */
+int msd_conv_relu_backward_bias(int dtype, int ndim, int64_t batch, int64_t c_out,
+                                const int64_t *spatial,
+                                const void *output, const int64_t *output_strides,
+                                const void *grad_output, const int64_t *grad_output_strides,
+                                void *grad_bias,
+                                void *workspace, int64_t workspace_bytes, void *stream);
+
+/* msd_conv_relu_backward_k and msd_conv_relu_backward_bias in one pass over the
+ * data: the two calls the dense block makes back to back for every layer
+ * (msd_block.py:113-126) share their reads of output and grad_output.
+ * grad_bias may be NULL. */
+int msd_conv_relu_backward_kb(int dtype, int ndim, int64_t batch, int64_t c_in, int64_t c_out,
+                              const int64_t *spatial, int dilation,
+                              const void *output, const int64_t *output_strides,
+                              const void *grad_output, const int64_t *grad_output_strides,
+                              const void *input, const int64_t *input_strides,
+                              void *grad_kernel, void *grad_bias,
+                              void *workspace, int64_t workspace_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MSD_HIP_H */

@@ -1,0 +1,282 @@
+// extern "C" entry points of libmsd_hip.so: argument checks, then dispatch to
+// the kernels.  Nothing here touches the device before the checks pass, so
+// every MSD_ERR_INVALID path can be exercised on a machine without a GPU.
+#include "../../include/msd_hip.h"
+#include "msd_kernels.h"
+
+#include <cstdarg>
+#include <cstdio>
+#include <string>
+
+namespace {
+
+thread_local std::string g_error;
+
+int fail(int code, const char *fmt, ...)
+{
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    g_error = buf;
+    return code;
+}
+
+int hip_fail(const char *where, hipError_t e)
+{
+    return fail(MSD_ERR_HIP, "%s: %s", where, hipGetErrorString(e));
+}
+
+// Geometry checks shared by all operators (rank, extents, dilation rule of
+// msd_custom_convolutions.cpp:39-52).  c_in may be 0 for the bias-only ops.
+int make_geom(const char *fn, int dtype, int ndim, int64_t batch, int64_t c_in, int64_t c_out,
+              const int64_t *spatial, int dilation, bool need_dilation, msd::Geom *g)
+{
+    if (dtype != MSD_F32 && dtype != MSD_F64) return fail(MSD_ERR_INVALID, "%s: dtype must be MSD_F32 or MSD_F64", fn);
+    if (ndim != 2 && ndim != 3) return fail(MSD_ERR_INVALID, "%s: expected 2 or 3 spatial dimensions, got %d", fn, ndim);
+    if (!spatial) return fail(MSD_ERR_INVALID, "%s: spatial is NULL", fn);
+    if (batch <= 0 || c_in < 0 || c_out <= 0)
+        return fail(MSD_ERR_INVALID, "%s: batch and channel counts must be positive", fn);
+    int64_t nvox = 1;
+    for (int i = 0; i < ndim; i++) {
+        if (spatial[i] <= 0) return fail(MSD_ERR_INVALID, "%s: spatial extents must be positive", fn);
+        nvox *= spatial[i];
+        if (nvox >= (int64_t(1) << 30)) return fail(MSD_ERR_INVALID, "%s: more than 2^30 voxels per channel", fn);
+    }
+    if (batch > 65535) return fail(MSD_ERR_INVALID, "%s: batch larger than 65535", fn);
+    if (c_in >= (1 << 20) || c_out >= (1 << 16)) return fail(MSD_ERR_INVALID, "%s: channel count too large", fn);
+    if (need_dilation) {
+        if (dilation <= 0) return fail(MSD_ERR_INVALID, "%s: Dilation must be 1 or greater", fn);
+        for (int i = 0; i < ndim; i++)
+            if (dilation > spatial[i])
+                return fail(MSD_ERR_INVALID, "%s: Dilation cannot be greater than size of image.", fn);
+    }
+    g->ndim = ndim;
+    g->B = (int)batch;
+    g->C = (int)c_in;
+    g->Wd = (int)c_out;
+    g->D = ndim == 3 ? (int)spatial[0] : 1;
+    g->H = (int)spatial[ndim - 2];
+    g->W = (int)spatial[ndim - 1];
+    g->dil = need_dilation ? dilation : 1;
+    g->nvox = (int)nvox;
+    return MSD_OK;
+}
+
+template <typename T>
+int make_view(const char *fn, const char *name, int ndim, const void *p, const int64_t *strides, msd::View<T> *v)
+{
+    if (!p) return fail(MSD_ERR_INVALID, "%s: %s is NULL", fn, name);
+    if (!strides) return fail(MSD_ERR_INVALID, "%s: %s_strides is NULL", fn, name);
+    for (int i = 0; i < ndim + 2; i++)
+        if (strides[i] < 0) return fail(MSD_ERR_INVALID, "%s: %s has a negative stride", fn, name);
+    v->p = (T *)p;
+    v->sb = strides[0];
+    v->sc = strides[1];
+    v->sz = ndim == 3 ? strides[2] : 0;
+    v->sy = strides[ndim];
+    v->sx = strides[ndim + 1];
+    return MSD_OK;
+}
+
+int check_workspace(const char *fn, const msd::Geom &g, size_t elem, const void *ws, int64_t bytes)
+{
+    const int64_t need = msd::generic_workspace_elems(g) * (int64_t)elem;
+    if (!ws || bytes < need)
+        return fail(MSD_ERR_WORKSPACE, "%s: workspace of %lld bytes needed, %lld given", fn, (long long)need,
+                    (long long)(ws ? bytes : 0));
+    return MSD_OK;
+}
+
+#define MSD_TRY(expr)            \
+    do {                         \
+        int rc_ = (expr);        \
+        if (rc_ != MSD_OK) return rc_; \
+    } while (0)
+
+template <typename T>
+int forward_t(const char *fn, bool relu, const msd::Geom &g, int ndim, const void *input, const int64_t *is,
+              const void *kernel, const void *bias, void *output, const int64_t *os, hipStream_t s)
+{
+    msd::View<const T> x;
+    msd::View<T> y;
+    MSD_TRY(make_view(fn, "input", ndim, input, is, &x));
+    MSD_TRY(make_view(fn, "output", ndim, output, os, &y));
+    if (!kernel) return fail(MSD_ERR_INVALID, "%s: kernel is NULL", fn);
+    if (!bias) return fail(MSD_ERR_INVALID, "%s: bias is NULL", fn);
+    hipError_t e = msd::generic_forward<T>(g, relu, x, (const T *)kernel, (const T *)bias, y, s);
+    return e == hipSuccess ? MSD_OK : hip_fail(fn, e);
+}
+
+int forward(const char *fn, bool relu, int dtype, int ndim, int64_t batch, int64_t c_in, int64_t c_out,
+            const int64_t *spatial, int dilation, const void *input, const int64_t *is, const void *kernel,
+            const void *bias, void *output, const int64_t *os, void *stream)
+{
+    msd::Geom g;
+    MSD_TRY(make_geom(fn, dtype, ndim, batch, c_in, c_out, spatial, dilation, true, &g));
+    if (c_in <= 0) return fail(MSD_ERR_INVALID, "%s: c_in must be positive", fn);
+    return dtype == MSD_F32
+               ? forward_t<float>(fn, relu, g, ndim, input, is, kernel, bias, output, os, (hipStream_t)stream)
+               : forward_t<double>(fn, relu, g, ndim, input, is, kernel, bias, output, os, (hipStream_t)stream);
+}
+
+template <typename T>
+int backward_x_t(const char *fn, bool relu, const msd::Geom &g, int ndim, const void *output, const int64_t *os,
+                 const void *grad_output, const int64_t *gs, const void *kernel, void *grad_input,
+                 const int64_t *xs, hipStream_t s)
+{
+    msd::View<const T> o{nullptr, 0, 0, 0, 0, 0}, gy;
+    msd::View<T> gx;
+    if (relu) MSD_TRY(make_view(fn, "output", ndim, output, os, &o));
+    MSD_TRY(make_view(fn, "grad_output", ndim, grad_output, gs, &gy));
+    MSD_TRY(make_view(fn, "grad_input", ndim, grad_input, xs, &gx));
+    if (!kernel) return fail(MSD_ERR_INVALID, "%s: kernel is NULL", fn);
+    hipError_t e = msd::generic_backward_x<T>(g, relu, o, gy, (const T *)kernel, gx, s);
+    return e == hipSuccess ? MSD_OK : hip_fail(fn, e);
+}
+
+int backward_x(const char *fn, bool relu, int dtype, int ndim, int64_t batch, int64_t c_in, int64_t c_out,
+               const int64_t *spatial, int dilation, const void *output, const int64_t *os, const void *grad_output,
+               const int64_t *gs, const void *kernel, void *grad_input, const int64_t *xs, void *stream)
+{
+    msd::Geom g;
+    MSD_TRY(make_geom(fn, dtype, ndim, batch, c_in, c_out, spatial, dilation, true, &g));
+    if (c_in <= 0) return fail(MSD_ERR_INVALID, "%s: c_in must be positive", fn);
+    return dtype == MSD_F32 ? backward_x_t<float>(fn, relu, g, ndim, output, os, grad_output, gs, kernel, grad_input,
+                                                  xs, (hipStream_t)stream)
+                            : backward_x_t<double>(fn, relu, g, ndim, output, os, grad_output, gs, kernel, grad_input,
+                                                   xs, (hipStream_t)stream);
+}
+
+template <typename T>
+int backward_kb_t(const char *fn, bool relu, const msd::Geom &g, int ndim, const void *output, const int64_t *os,
+                  const void *grad_output, const int64_t *gs, const void *input, const int64_t *xs, void *grad_kernel,
+                  void *grad_bias, void *ws, int64_t ws_bytes, hipStream_t s)
+{
+    msd::View<const T> o{nullptr, 0, 0, 0, 0, 0}, gy, x{nullptr, 0, 0, 0, 0, 0};
+    if (relu) MSD_TRY(make_view(fn, "output", ndim, output, os, &o));
+    MSD_TRY(make_view(fn, "grad_output", ndim, grad_output, gs, &gy));
+    if (grad_kernel) MSD_TRY(make_view(fn, "input", ndim, input, xs, &x));
+    if (!grad_kernel && !grad_bias) return fail(MSD_ERR_INVALID, "%s: no gradient buffer given", fn);
+    MSD_TRY(check_workspace(fn, g, sizeof(T), ws, ws_bytes));
+    hipError_t e = msd::generic_backward_kb<T>(g, relu, o, gy, x, (T *)grad_kernel, (T *)grad_bias, (T *)ws, s);
+    return e == hipSuccess ? MSD_OK : hip_fail(fn, e);
+}
+
+int backward_kb(const char *fn, bool relu, bool need_k, int dtype, int ndim, int64_t batch, int64_t c_in,
+                int64_t c_out, const int64_t *spatial, int dilation, const void *output, const int64_t *os,
+                const void *grad_output, const int64_t *gs, const void *input, const int64_t *xs, void *grad_kernel,
+                void *grad_bias, void *ws, int64_t ws_bytes, void *stream)
+{
+    msd::Geom g;
+    MSD_TRY(make_geom(fn, dtype, ndim, batch, c_in, c_out, spatial, dilation, need_k, &g));
+    if (need_k && c_in <= 0) return fail(MSD_ERR_INVALID, "%s: c_in must be positive", fn);
+    if (need_k && !grad_kernel) return fail(MSD_ERR_INVALID, "%s: grad_kernel is NULL", fn);
+    return dtype == MSD_F32 ? backward_kb_t<float>(fn, relu, g, ndim, output, os, grad_output, gs, input, xs,
+                                                   grad_kernel, grad_bias, ws, ws_bytes, (hipStream_t)stream)
+                            : backward_kb_t<double>(fn, relu, g, ndim, output, os, grad_output, gs, input, xs,
+                                                    grad_kernel, grad_bias, ws, ws_bytes, (hipStream_t)stream);
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *msd_last_error(void) { return g_error.c_str(); }
+
+int msd_abi_version(void) { return 1; }
+
+int64_t msd_workspace_bytes(int dtype, int ndim, int64_t batch, int64_t c_in, int64_t c_out, const int64_t *spatial)
+{
+    msd::Geom g;
+    if (make_geom("msd_workspace_bytes", dtype, ndim, batch, c_in, c_out, spatial, 1, false, &g) != MSD_OK) return -1;
+    return msd::generic_workspace_elems(g) * (dtype == MSD_F32 ? 4 : 8);
+}
+
+int msd_conv_forward(int dtype, int ndim, int64_t batch, int64_t c_in, int64_t c_out, const int64_t *spatial,
+                     int dilation, const void *input, const int64_t *input_strides, const void *kernel,
+                     const void *bias, void *output, const int64_t *output_strides, void *stream)
+{
+    return forward("conv_forward", false, dtype, ndim, batch, c_in, c_out, spatial, dilation, input, input_strides,
+                   kernel, bias, output, output_strides, stream);
+}
+
+int msd_conv_relu_forward(int dtype, int ndim, int64_t batch, int64_t c_in, int64_t c_out, const int64_t *spatial,
+                          int dilation, const void *input, const int64_t *input_strides, const void *kernel,
+                          const void *bias, void *output, const int64_t *output_strides, void *stream)
+{
+    return forward("conv_relu_forward", true, dtype, ndim, batch, c_in, c_out, spatial, dilation, input,
+                   input_strides, kernel, bias, output, output_strides, stream);
+}
+
+int msd_conv_backward_x(int dtype, int ndim, int64_t batch, int64_t c_in, int64_t c_out, const int64_t *spatial,
+                        int dilation, const void *grad_output, const int64_t *grad_output_strides, const void *kernel,
+                        void *grad_input, const int64_t *grad_input_strides, void *stream)
+{
+    return backward_x("conv_backward_x", false, dtype, ndim, batch, c_in, c_out, spatial, dilation, nullptr, nullptr,
+                      grad_output, grad_output_strides, kernel, grad_input, grad_input_strides, stream);
+}
+
+int msd_conv_relu_backward_x(int dtype, int ndim, int64_t batch, int64_t c_in, int64_t c_out, const int64_t *spatial,
+                             int dilation, const void *output, const int64_t *output_strides, const void *grad_output,
+                             const int64_t *grad_output_strides, const void *kernel, void *grad_input,
+                             const int64_t *grad_input_strides, void *stream)
+{
+    return backward_x("conv_relu_backward_x", true, dtype, ndim, batch, c_in, c_out, spatial, dilation, output,
+                      output_strides, grad_output, grad_output_strides, kernel, grad_input, grad_input_strides, stream);
+}
+
+int msd_conv_backward_k(int dtype, int ndim, int64_t batch, int64_t c_in, int64_t c_out, const int64_t *spatial,
+                        int dilation, const void *grad_output, const int64_t *grad_output_strides, const void *input,
+                        const int64_t *input_strides, void *grad_kernel, void *workspace, int64_t workspace_bytes,
+                        void *stream)
+{
+    return backward_kb("conv_backward_k", false, true, dtype, ndim, batch, c_in, c_out, spatial, dilation, nullptr,
+                       nullptr, grad_output, grad_output_strides, input, input_strides, grad_kernel, nullptr,
+                       workspace, workspace_bytes, stream);
+}
+
+int msd_conv_relu_backward_k(int dtype, int ndim, int64_t batch, int64_t c_in, int64_t c_out, const int64_t *spatial,
+                             int dilation, const void *output, const int64_t *output_strides, const void *grad_output,
+                             const int64_t *grad_output_strides, const void *input, const int64_t *input_strides,
+                             void *grad_kernel, void *workspace, int64_t workspace_bytes, void *stream)
+{
+    return backward_kb("conv_relu_backward_k", true, true, dtype, ndim, batch, c_in, c_out, spatial, dilation, output,
+                       output_strides, grad_output, grad_output_strides, input, input_strides, grad_kernel, nullptr,
+                       workspace, workspace_bytes, stream);
+}
+
+int msd_conv_backward_bias(int dtype, int ndim, int64_t batch, int64_t c_out, const int64_t *spatial,
+                           const void *grad_output, const int64_t *grad_output_strides, void *grad_bias,
+                           void *workspace, int64_t workspace_bytes, void *stream)
+{
+    if (!grad_bias) return fail(MSD_ERR_INVALID, "conv_backward_bias: grad_bias is NULL");
+    return backward_kb("conv_backward_bias", false, false, dtype, ndim, batch, 0, c_out, spatial, 1, nullptr, nullptr,
+                       grad_output, grad_output_strides, nullptr, nullptr, nullptr, grad_bias, workspace,
+                       workspace_bytes, stream);
+}
+
+int msd_conv_relu_backward_bias(int dtype, int ndim, int64_t batch, int64_t c_out, const int64_t *spatial,
+                                const void *output, const int64_t *output_strides, const void *grad_output,
+                                const int64_t *grad_output_strides, void *grad_bias, void *workspace,
+                                int64_t workspace_bytes, void *stream)
+{
+    if (!grad_bias) return fail(MSD_ERR_INVALID, "conv_relu_backward_bias: grad_bias is NULL");
+    return backward_kb("conv_relu_backward_bias", true, false, dtype, ndim, batch, 0, c_out, spatial, 1, output,
+                       output_strides, grad_output, grad_output_strides, nullptr, nullptr, nullptr, grad_bias,
+                       workspace, workspace_bytes, stream);
+}
+
+int msd_conv_relu_backward_kb(int dtype, int ndim, int64_t batch, int64_t c_in, int64_t c_out, const int64_t *spatial,
+                              int dilation, const void *output, const int64_t *output_strides, const void *grad_output,
+                              const int64_t *grad_output_strides, const void *input, const int64_t *input_strides,
+                              void *grad_kernel, void *grad_bias, void *workspace, int64_t workspace_bytes,
+                              void *stream)
+{
+    return backward_kb("conv_relu_backward_kb", true, true, dtype, ndim, batch, c_in, c_out, spatial, dilation, output,
+                       output_strides, grad_output, grad_output_strides, input, input_strides, grad_kernel, grad_bias,
+                       workspace, workspace_bytes, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,132 @@
+"""Mixed-scale dense block: ``depth`` dilated conv+ReLU layers that all write
+into ONE growing channel stack; layer ``i`` reads every channel in front of it.
+
+API of the reference's msd_block.py: ``MSDBlockFunction(input, dilations, bias,
+*weights)`` (:8-134), ``msd_block``, ``MSDBlock``/``MSDBlock2d``/``MSDBlock3d``
+with parameters ``weight{i}`` of shape ``(width, c_in + width*i, 3, 3[, 3])``
+and one flat ``bias`` of ``depth * width`` (:140-249), so checkpoints are
+interchangeable.
+"""
+import math
+
+import torch
+
+from . import msd_custom_convolutions as cc
+
+
+class MSDBlockFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, input, dilations, bias, *weights):
+        if len(dilations) != len(weights):
+            raise AssertionError("number of weights does not match depth")
+        if input.dim() not in (4, 5):
+            raise ValueError("Input to MSDBlock must be 2D or 3D")
+        widths = [w.shape[0] for w in weights]
+        if len(bias) != sum(widths):
+            raise AssertionError("number of biases does not match number of output channels from weights")
+
+        c_in = input.shape[1]
+        stack = input.new_empty(input.shape[0], c_in + sum(widths), *input.shape[2:])
+        stack[:, :c_in] = input
+
+        first, b0 = c_in, 0
+        for weight, width, dilation in zip(weights, widths, dilations):
+            cc.conv_relu_forward(stack[:, :first], weight, bias[b0:b0 + width],
+                                 stack[:, first:first + width], dilation)
+            first += width
+            b0 += width
+
+        ctx.dilations = tuple(dilations)
+        ctx.save_for_backward(bias, stack, *weights)
+        return stack
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        bias, stack, *weights = ctx.saved_tensors
+        if grad_output.dim() != stack.dim():
+            raise AssertionError("Mismatched tensor dimensions.")
+        need_input, _, need_bias, *need_weights = ctx.needs_input_grad
+
+        # Working copy of the incoming gradient: layer idx adds its input
+        # gradient to channels [0, first), which later iterations consume.
+        grads = grad_output.clone()
+        grad_bias = torch.zeros_like(bias)
+        grad_weights = [None] * len(weights)
+
+        last, b1 = stack.shape[1], bias.shape[0]
+        for idx in reversed(range(len(weights))):
+            weight = weights[idx]
+            width = weight.shape[0]
+            first, b0 = last - width, b1 - width
+            out_i, gout_i = stack[:, first:last], grads[:, first:last]
+            dilation = ctx.dilations[idx]
+
+            if idx > 0 or need_input:
+                cc.conv_relu_backward_x(out_i, gout_i, weight, grads[:, :first], dilation)
+            if need_weights[idx]:
+                grad_weights[idx] = torch.zeros_like(weight)
+                cc.conv_relu_backward_kb(out_i, gout_i, stack[:, :first], grad_weights[idx],
+                                         grad_bias[b0:b1] if need_bias else None, dilation)
+            elif need_bias:
+                cc.conv_relu_backward_bias(out_i, gout_i, grad_bias[b0:b1])
+            last, b1 = first, b0
+
+        grad_input = grads[:, :weights[0].shape[1]] if need_input else None
+        return (grad_input, None, grad_bias if need_bias else None, *grad_weights)
+
+
+msd_block = MSDBlockFunction.apply
+
+
+class MSDBlock(torch.nn.Module):
+    def __init__(self, in_channels, dilations, width=1, ndim=2):
+        """Mixed-scale dense block.
+
+        in_channels : number of input channels
+        dilations   : one dilation per layer (its length is the depth)
+        width       : output channels per layer
+        ndim        : 2 or 3
+
+        The output has ``in_channels + len(dilations) * width`` channels: the
+        input followed by every layer's output.
+        """
+        super().__init__()
+        if ndim not in (2, 3):
+            raise ValueError("ndim must be 2 or 3")
+        self.kernel_size = (3,) * ndim
+        self.width = width
+        self.dilations = dilations
+
+        depth = len(dilations)
+        self.bias = torch.nn.Parameter(torch.empty(depth * width))
+        self.weights = []
+        for i in range(depth):
+            weight = torch.nn.Parameter(torch.empty(width, in_channels + width * i, *self.kernel_size))
+            self.register_parameter(f"weight{i}", weight)
+            self.weights.append(weight)
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        # same draws, in the same order, as msd_block.py:183-191
+        for weight in self.weights:
+            torch.nn.init.kaiming_uniform_(weight, a=math.sqrt(5))
+        fan_in, _ = torch.nn.init._calculate_fan_in_and_fan_out(self.weights[0])
+        bound = 1 / math.sqrt(fan_in)
+        torch.nn.init.uniform_(self.bias, -bound, bound)
+
+    def forward(self, input):
+        # Look the weights up by attribute on every call: after a device move,
+        # a DataParallel replication or torch.nn.utils.prune the list made in
+        # __init__ may hold stale tensors (msd_block.py:193-209).
+        weights = (getattr(self, f"weight{i}") for i in range(len(self.weights)))
+        return msd_block(input, self.dilations, self.bias, *weights)
+
+
+class MSDBlock2d(MSDBlock):
+    def __init__(self, in_channels, dilations, width=1):
+        super().__init__(in_channels, dilations, width=width, ndim=2)
+
+
+class MSDBlock3d(MSDBlock):
+    def __init__(self, in_channels, dilations, width=1):
+        super().__init__(in_channels, dilations, width=width, ndim=3)

@@ -1,0 +1,288 @@
+"""The eight operators of the reference's native module, on MI355X.
+
+Drop-in for the pybind11 module ``msd_custom_convolutions`` of the reference
+(msd_custom_convolutions.cpp:343-369): same function names, same positional
+arguments, same in-place semantics, ``RuntimeError`` on every invalid call.
+The tensors' device pointers, sizes and strides are handed to the C ABI of
+``libmsd_hip.so`` on torch's current stream; no tensor is copied or retained.
+
+``block_size`` is accepted for compatibility and ignored: the launch shapes are
+chosen by the library for gfx950.
+"""
+import ctypes
+
+import torch
+
+from . import _native
+
+_DTYPES = {torch.float32: _native.MSD_F32, torch.float64: _native.MSD_F64}
+
+
+def _fail(fn, msg):
+    raise RuntimeError(f"{fn}: {msg}")
+
+
+def _check_same_gpu(fn, named):
+    """torch::checkAllSameGPU (msd_custom_convolutions.cpp:98)."""
+    first = named[0][1]
+    for name, t in named:
+        if not isinstance(t, torch.Tensor):
+            raise TypeError(f"{fn}: argument '{name}' must be a torch.Tensor")
+        if not t.is_cuda:
+            _fail(fn, f"Expected tensor for argument '{name}' to be on a GPU, but it is on {t.device}")
+        if t.device != first.device:
+            _fail(fn, f"Expected all tensors on the same GPU, but '{name}' is on {t.device} "
+                      f"and '{named[0][0]}' is on {first.device}")
+
+
+def _check_same_type(fn, named):
+    """torch::checkAllSameType (msd_custom_convolutions.cpp:99)."""
+    first = named[0][1]
+    for name, t in named:
+        if t.dtype != first.dtype:
+            _fail(fn, f"Expected '{name}' to have the same type as '{named[0][0]}' "
+                      f"({first.dtype}), but it has {t.dtype}")
+    if first.dtype not in _DTYPES:
+        _fail(fn, f"only float32 and float64 are supported, got {first.dtype}")
+
+
+def _check_in_out_shape(fn, a, b):
+    """checkInOutShape (msd_custom_convolutions.cpp:68-83)."""
+    if a.dim() != b.dim():
+        _fail(fn, f"tensors must have the same number of dimensions, got {a.dim()} and {b.dim()}")
+    if a.dim() not in (4, 5):
+        _fail(fn, f"expected a 4- or 5-dimensional tensor, got {a.dim()} dimensions")
+    if a.shape[0] != b.shape[0]:
+        _fail(fn, "Input batch dimension does not match output batch dimension. ")
+    if tuple(a.shape[2:]) != tuple(b.shape[2:]):
+        _fail(fn, "Input shape does not match output shape. ")
+
+
+def _check_kernel(fn, kernel):
+    """checkKernel3x3 + checkContiguous (msd_custom_convolutions.cpp:25-37,100)."""
+    if kernel.dim() not in (4, 5):
+        _fail(fn, "Expected 4 or 5 dimensional kernel.")
+    if any(s != 3 for s in kernel.shape[2:]):
+        _fail(fn, "Kernel shape must be 3x3" if kernel.dim() == 4 else "Kernel shape must be 3x3x3")
+    if not kernel.is_contiguous():
+        _fail(fn, "Expected kernel to be contiguous")
+
+
+def _check_dim(fn, name, t, dim):
+    if t.dim() != dim:
+        _fail(fn, f"Expected {dim}-dimensional tensor for '{name}', but got {t.dim()} dimensions")
+
+
+def _check_dilation(fn, t, dilation):
+    """checkDilation (msd_custom_convolutions.cpp:39-52)."""
+    if not isinstance(dilation, int) or isinstance(dilation, bool):
+        raise TypeError(f"{fn}: dilation must be an int")
+    if dilation <= 0:
+        _fail(fn, "Dilation must be 1 or greater")
+    if any(dilation > s for s in t.shape[2:]):
+        _fail(fn, "Dilation cannot be greater than size of image. ")
+
+
+def _check_block_size(fn, block_size):
+    if block_size is None:
+        return
+    if len(tuple(block_size)) != 3:
+        raise TypeError(f"{fn}: block_size must be a tuple of three ints (z, y, x)")
+
+
+def _head(data, c_in, c_out, dilation):
+    """dtype, ndim, batch, c_in, c_out, spatial, dilation."""
+    return (_DTYPES[data.dtype], data.dim() - 2, data.shape[0], c_in, c_out,
+            _native.i64_array(tuple(data.shape[2:])), dilation)
+
+
+def _view(t):
+    return ctypes.c_void_p(t.data_ptr()), _native.i64_array(t.stride())
+
+
+def _stream(t):
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _workspace(data, c_in, c_out):
+    lib = _native.load()
+    need = lib.msd_workspace_bytes(_DTYPES[data.dtype], data.dim() - 2, data.shape[0], c_in, c_out,
+                                   _native.i64_array(tuple(data.shape[2:])))
+    if need < 0:
+        _fail("workspace", _native.last_error())
+    ws = torch.empty(max(int(need), 8), dtype=torch.uint8, device=data.device)
+    return ws, ctypes.c_void_p(ws.data_ptr()), int(need)
+
+
+def _call(fn_name, device, *args):
+    lib = _native.load()
+    with torch.cuda.device(device):
+        rc = getattr(lib, fn_name)(*args)
+    if rc != _native.MSD_OK:
+        raise RuntimeError(_native.last_error())
+
+
+def _forward(fn, native, input, kernel, bias, output, dilation, block_size):
+    _check_same_gpu(fn, [("input", input), ("kernel", kernel), ("bias", bias), ("output", output)])
+    _check_same_type(fn, [("input", input), ("kernel", kernel), ("bias", bias), ("output", output)])
+    _check_kernel(fn, kernel)
+    _check_in_out_shape(fn, input, output)
+    for name, t in (("input", input), ("kernel", kernel), ("output", output)):
+        _check_dim(fn, name, t, kernel.dim())
+    _check_dim(fn, "bias", bias, 1)
+    if kernel.shape[1] != input.shape[1]:
+        _fail(fn, "Kernel shape does not match input channels. ")
+    if kernel.shape[0] != output.shape[1]:
+        _fail(fn, "Kernel shape does not match output channels. ")
+    if bias.shape[0] != output.shape[1]:
+        _fail(fn, "Bias shape does not match output channels. ")
+    _check_dilation(fn, input, dilation)
+    _check_block_size(fn, block_size)
+    bias = bias.contiguous()
+    _call(native, input.device, *_head(input, input.shape[1], output.shape[1], dilation), *_view(input),
+          ctypes.c_void_p(kernel.data_ptr()), ctypes.c_void_p(bias.data_ptr()), *_view(output), _stream(input))
+
+
+def conv_forward(input, kernel, bias, output, dilation, block_size=None):
+    """output = bias + conv(input) (msd_custom_convolutions.cpp:85-117)."""
+    _forward("conv_forward", "msd_conv_forward", input, kernel, bias, output, dilation, block_size)
+
+
+def conv_relu_forward(input, kernel, bias, output, dilation, block_size=None):
+    """output = max(0, bias + conv(input)) (msd_custom_convolutions.cpp:213-245)."""
+    _forward("conv_relu_forward", "msd_conv_relu_forward", input, kernel, bias, output, dilation, block_size)
+
+
+def _backward_x(fn, native, output, grad_output, kernel, grad_input, dilation, block_size):
+    relu = output is not None
+    named = [("grad_input", grad_input), ("kernel", kernel)]
+    if relu:
+        named.append(("output", output))
+    named.append(("grad_output", grad_output))
+    _check_same_gpu(fn, named)
+    _check_same_type(fn, named)
+    _check_kernel(fn, kernel)
+    _check_in_out_shape(fn, grad_input, grad_output)
+    if relu:
+        _check_in_out_shape(fn, grad_input, output)
+    for name, t in named:
+        _check_dim(fn, name, t, kernel.dim())
+    if kernel.shape[1] != grad_input.shape[1]:
+        _fail(fn, "Kernel shape does not match input channels. ")
+    if kernel.shape[0] != grad_output.shape[1] or (relu and kernel.shape[0] != output.shape[1]):
+        _fail(fn, "Kernel shape does not match output channels. ")
+    _check_dilation(fn, grad_input, dilation)
+    _check_block_size(fn, block_size)
+    head = _head(grad_input, grad_input.shape[1], grad_output.shape[1], dilation)
+    views = (*_view(output),) if relu else ()
+    _call(native, grad_input.device, *head, *views, *_view(grad_output), ctypes.c_void_p(kernel.data_ptr()),
+          *_view(grad_input), _stream(grad_input))
+
+
+def conv_backward_x(grad_output, kernel, grad_input, dilation, block_size=None):
+    """grad_input += conv^T(grad_output) (msd_custom_convolutions.cpp:119-148)."""
+    _backward_x("conv_backward_x", "msd_conv_backward_x", None, grad_output, kernel, grad_input, dilation,
+                block_size)
+
+
+def conv_relu_backward_x(output, grad_output, kernel, grad_input, dilation, block_size=None):
+    """grad_input += conv^T(grad_output * [output > 0]) (msd_custom_convolutions.cpp:247-281)."""
+    _backward_x("conv_relu_backward_x", "msd_conv_relu_backward_x", output, grad_output, kernel, grad_input,
+                dilation, block_size)
+
+
+def _backward_k(fn, native, output, grad_output, input, grad_kernel, grad_bias, dilation, block_size):
+    relu = output is not None
+    named = [("input", input), ("grad_kernel", grad_kernel)]
+    if relu:
+        named.append(("output", output))
+    named.append(("grad_output", grad_output))
+    if grad_bias is not None:
+        named.append(("grad_bias", grad_bias))
+    _check_same_gpu(fn, named)
+    _check_same_type(fn, named)
+    _check_kernel(fn, grad_kernel)
+    _check_in_out_shape(fn, input, grad_output)
+    if relu:
+        _check_in_out_shape(fn, input, output)
+    for name, t in named:
+        if name != "grad_bias":
+            _check_dim(fn, name, t, grad_kernel.dim())
+    if grad_kernel.shape[1] != input.shape[1]:
+        _fail(fn, "Kernel shape does not match input channels. ")
+    if grad_kernel.shape[0] != grad_output.shape[1] or (relu and grad_kernel.shape[0] != output.shape[1]):
+        _fail(fn, "Kernel shape does not match output channels. ")
+    if grad_bias is not None:
+        _check_dim(fn, "grad_bias", grad_bias, 1)
+        if grad_bias.shape[0] != grad_output.shape[1]:
+            _fail(fn, "Bias shape does not match output channels. ")
+        if not grad_bias.is_contiguous():
+            _fail(fn, "Expected grad_bias to be contiguous")
+    _check_dilation(fn, input, dilation)
+    _check_block_size(fn, block_size)
+    c_in, c_out = input.shape[1], grad_output.shape[1]
+    ws, ws_ptr, ws_bytes = _workspace(input, c_in, c_out)
+    head = _head(input, c_in, c_out, dilation)
+    views = (*_view(output),) if relu else ()
+    grads = (ctypes.c_void_p(grad_kernel.data_ptr()),)
+    if native == "msd_conv_relu_backward_kb":
+        grads += (ctypes.c_void_p(grad_bias.data_ptr() if grad_bias is not None else 0),)
+    _call(native, input.device, *head, *views, *_view(grad_output), *_view(input), *grads, ws_ptr, ws_bytes,
+          _stream(input))
+
+
+def conv_backward_k(grad_output, input, grad_kernel, dilation, block_size=None):
+    """grad_kernel += d/dkernel (msd_custom_convolutions.cpp:150-178)."""
+    _backward_k("conv_backward_k", "msd_conv_backward_k", None, grad_output, input, grad_kernel, None, dilation,
+                block_size)
+
+
+def conv_relu_backward_k(output, grad_output, input, grad_kernel, dilation, block_size=None):
+    """grad_kernel += d/dkernel with the ReLU mask (msd_custom_convolutions.cpp:283-316)."""
+    _backward_k("conv_relu_backward_k", "msd_conv_relu_backward_k", output, grad_output, input, grad_kernel, None,
+                dilation, block_size)
+
+
+def conv_relu_backward_kb(output, grad_output, input, grad_kernel, grad_bias, dilation, block_size=None):
+    """conv_relu_backward_k and conv_relu_backward_bias in one pass (the pair of
+    calls msd_block.py:113-126 makes per layer).  Not part of the reference's module."""
+    _backward_k("conv_relu_backward_kb", "msd_conv_relu_backward_kb", output, grad_output, input, grad_kernel,
+                grad_bias, dilation, block_size)
+
+
+def _backward_bias(fn, native, output, grad_output, grad_bias, block_size):
+    relu = output is not None
+    named = [("grad_bias", grad_bias)]
+    if relu:
+        named.append(("output", output))
+    named.append(("grad_output", grad_output))
+    _check_same_gpu(fn, named)
+    _check_same_type(fn, named)
+    if relu:
+        _check_in_out_shape(fn, output, grad_output)
+    elif grad_output.dim() not in (4, 5):
+        _fail(fn, f"expected a 4- or 5-dimensional tensor, got {grad_output.dim()} dimensions")
+    _check_dim(fn, "grad_bias", grad_bias, 1)
+    if grad_bias.shape[0] != grad_output.shape[1]:
+        _fail(fn, "Bias shape does not match output channels. ")
+    if not grad_bias.is_contiguous():
+        _fail(fn, "Expected grad_bias to be contiguous")
+    _check_block_size(fn, block_size)
+    c_out = grad_output.shape[1]
+    ws, ws_ptr, ws_bytes = _workspace(grad_output, 0, c_out)
+    head = (_DTYPES[grad_output.dtype], grad_output.dim() - 2, grad_output.shape[0], c_out,
+            _native.i64_array(tuple(grad_output.shape[2:])))
+    views = (*_view(output),) if relu else ()
+    _call(native, grad_output.device, *head, *views, *_view(grad_output), ctypes.c_void_p(grad_bias.data_ptr()),
+          ws_ptr, ws_bytes, _stream(grad_output))
+
+
+def conv_backward_bias(grad_output, grad_bias, block_size=None):
+    """grad_bias += grad_output summed over batch and voxels (msd_custom_convolutions.cpp:180-211)."""
+    _backward_bias("conv_backward_bias", "msd_conv_backward_bias", None, grad_output, grad_bias, block_size)
+
+
+def conv_relu_backward_bias(output, grad_output, grad_bias, block_size=None):
+    """grad_bias += grad_output summed where output > 0 (msd_custom_convolutions.cpp:318-338)."""
+    _backward_bias("conv_relu_backward_bias", "msd_conv_relu_backward_bias", output, grad_output, grad_bias,
+                   block_size)

@@ -1,0 +1,81 @@
+"""MSD network module: dense block + final 1x1 layer (reference msd_module.py)."""
+from math import sqrt
+
+import torch
+
+from .msd_block import MSDBlock
+
+
+def units_in_front(c_in, width, layer_depth):
+    """Number of channels that hidden layer ``layer_depth`` (zero-based) reads:
+    the network inputs plus the outputs of every earlier layer."""
+    return c_in + width * layer_depth
+
+
+def init_convolution_weights(conv_weight, c_in, c_out, width, depth):
+    """Normal(0, sqrt(2 / n)) initialisation of Pelt & Sethian (PNAS 115(2), 2018),
+    with n = taps * (c_in + width * (depth - 1)) + c_out, as msd_module.py:27-57."""
+    taps = 1
+    for s in conv_weight.shape[2:]:
+        taps *= s
+    n = taps * (c_in + width * (depth - 1)) + c_out
+    conv_weight.normal_(0, sqrt(2 / n))
+
+
+class MSDFinalLayer(torch.nn.Module):
+    """1x1 convolution over the whole channel stack, zero-initialised.
+
+    Stored as ``linear = Conv1d(c_in, c_out, 1)`` acting on a (B, C, voxels)
+    view, which keeps the state-dict keys of msd_module.py:60-88."""
+
+    def __init__(self, c_in, c_out):
+        super().__init__()
+        self.c_in = c_in
+        self.c_out = c_out
+        self.linear = torch.nn.Conv1d(c_in, c_out, 1)
+        self.reset_parameters()
+
+    def forward(self, input):
+        b, c, *size = input.shape
+        flat = input.view(b, c, -1)
+        return self.linear(flat).view(b, self.c_out, *size)
+
+    def reset_parameters(self):
+        self.linear.weight.data.zero_()
+        self.linear.bias.data.zero_()
+
+
+class MSDModule(torch.nn.Module):
+    def __init__(self, c_in, c_out, depth, width, dilations=[1, 2, 3, 4, 5, 6, 7, 8, 9, 10], ndim=2):
+        """Mixed-scale dense network.
+
+        c_in, c_out : input / output channels
+        depth       : number of hidden layers
+        width       : channels per hidden layer
+        dilations   : list of dilations, repeated cyclically over the layers
+                      (default 1..10; [1, 2, 4, 8] is a common alternative)
+        ndim        : 2 or 3
+        """
+        super().__init__()
+        if depth < 1:
+            raise ValueError(f"Depth must be at least 1. Got: {depth}.")
+        if width < 1:
+            raise ValueError(f"Width must be at least 1. Got: {width}.")
+        self.c_in = c_in
+        self.c_out = c_out
+        self.depth = depth
+        self.width = width
+        self.dilations = [dilations[i % len(dilations)] for i in range(depth)]
+
+        self.msd_block = MSDBlock(c_in, self.dilations, width, ndim=ndim)
+        self.final_layer = MSDFinalLayer(c_in=c_in + width * depth, c_out=c_out)
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        for w in self.msd_block.weights:
+            init_convolution_weights(w.data, self.c_in, self.c_out, self.width, self.depth)
+        self.msd_block.bias.data.zero_()
+        self.final_layer.reset_parameters()
+
+    def forward(self, input):
+        return self.final_layer(self.msd_block(input))

@@ -1,0 +1,35 @@
+"""MSD network for segmentation (reference msd_segmentation_model.py:10-119)."""
+import torch.nn as nn
+
+from .msd_model import MSDModel, _moments, scaling_module_set_bias, scaling_module_set_scale
+
+
+class MSDSegmentationModel(MSDModel):
+    def __init__(self, c_in, num_labels, depth, width, *, dilations=[1, 2, 3, 4, 5, 6, 7, 8, 9, 10],
+                 parallel=False, ndim=2):
+        """``num_labels`` output classes; log-softmax over channels + NLL loss."""
+        self.num_labels = num_labels
+        super().__init__(c_in, num_labels, depth, width, dilations, ndim=ndim)
+        self.criterion = nn.NLLLoss()
+
+        net_trained = nn.Sequential(self.msd, nn.LogSoftmax(dim=1))
+        self.net = nn.Sequential(self.scale_in, net_trained)
+        self.net.cuda()
+        if parallel:
+            self.net = nn.DataParallel(self.net)
+        self.init_optimizer(net_trained)
+
+    def set_normalization(self, dataloader):
+        """Only the input is normalised; the targets are labels."""
+        mean, std = _moments(d[0] for d in dataloader)
+        scaling_module_set_scale(self.scale_in, 1 / std)
+        scaling_module_set_bias(self.scale_in, -mean / std)
+
+    def set_target(self, target):
+        target = target.long()
+        lo, hi = target.min(), target.max()
+        if lo < 0 or self.num_labels <= hi:
+            raise ValueError(
+                f"Target invalid: expected values in range {[0, self.num_labels - 1]}, but got {[lo, hi]}")
+        # NLLLoss takes (B, *spatial) class indices: drop the channel axis
+        self.target = target.squeeze(1).cuda()

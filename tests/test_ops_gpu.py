@@ -1,0 +1,141 @@
+"""Parity of the HIP operators (called through the C ABI of libmsd_hip.so via
+msd_pytorch_amd.msd_custom_convolutions) with the CPU oracle on identical
+seeded inputs.
+
+Tolerances (max |diff| / max |ref|): fp32 forward 1e-5, fp32 gradients 1e-4
+(their summation order differs from the oracle's), fp64 1e-11."""
+import pytest
+import torch
+
+import oracle
+from cases import ALL_SHAPES, SHAPES_FAST, make_problem, rel_err
+
+pytestmark = pytest.mark.gpu
+
+TOL_FWD = {torch.float32: 1e-5, torch.float64: 1e-11}
+TOL_GRAD = {torch.float32: 1e-4, torch.float64: 1e-11}
+
+
+@pytest.fixture(scope="module")
+def cc():
+    from msd_pytorch_amd import msd_custom_convolutions
+    return msd_custom_convolutions
+
+
+def run_all(ops, p, relu):
+    """forward, backward_x (accumulating into noise), backward_k, backward_bias."""
+    gk = torch.zeros_like(p["k"])
+    gb = torch.zeros_like(p["bias"])
+    if relu:
+        ops.conv_relu_forward(p["x"], p["k"], p["bias"], p["y"], p["d"])
+        ops.conv_relu_backward_x(p["y"], p["gy"], p["k"], p["gx"], p["d"])
+        ops.conv_relu_backward_k(p["y"], p["gy"], p["x"], gk, p["d"])
+        ops.conv_relu_backward_bias(p["y"], p["gy"], gb)
+    else:
+        ops.conv_forward(p["x"], p["k"], p["bias"], p["y"], p["d"])
+        ops.conv_backward_x(p["gy"], p["k"], p["gx"], p["d"])
+        ops.conv_backward_k(p["gy"], p["x"], gk, p["d"])
+        ops.conv_backward_bias(p["gy"], gb)
+    return gk, gb
+
+
+def check_case(cc, shape, dtype, relu):
+    ref = make_problem(shape, dtype)
+    dev = make_problem(shape, dtype, device="cuda")
+    want_gk, want_gb = run_all(oracle, ref, relu)
+    got_gk, got_gb = run_all(cc, dev, relu)
+    torch.cuda.synchronize()
+    # the whole stack: the input channels must be untouched, the output channels match
+    assert rel_err(dev["stack"], ref["stack"]) <= TOL_FWD[dtype], "forward"
+    assert torch.equal(dev["x"].cpu(), ref["x"]), "forward wrote outside its output channels"
+    assert rel_err(dev["gstack"], ref["gstack"]) <= TOL_GRAD[dtype], "backward_x"
+    assert torch.equal(dev["gy"].cpu(), ref["gy"]), "backward_x wrote outside grad_input"
+    assert rel_err(got_gk, want_gk) <= TOL_GRAD[dtype], "backward_k"
+    assert rel_err(got_gb, want_gb) <= TOL_GRAD[dtype], "backward_bias"
+
+
+@pytest.mark.parametrize("relu", [1, 0])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("shape", ALL_SHAPES)
+def test_small_shapes(cc, shape, dtype, relu):
+    check_case(cc, shape, dtype, relu)
+
+
+@pytest.mark.parametrize("relu", [1, 0])
+@pytest.mark.parametrize("shape", SHAPES_FAST)
+def test_larger_shapes_f32(cc, shape, relu):
+    check_case(cc, shape, torch.float32, relu)
+
+
+@pytest.mark.parametrize("shape", [SHAPES_FAST[1], SHAPES_FAST[7]])
+def test_larger_shapes_f64(cc, shape):
+    check_case(cc, shape, torch.float64, 1)
+
+
+def test_fused_weight_and_bias_gradient(cc):
+    for shape in (SHAPES_FAST[3], SHAPES_FAST[8]):
+        p = make_problem(shape, torch.float32, device="cuda")
+        cc.conv_relu_forward(p["x"], p["k"], p["bias"], p["y"], p["d"])
+        gk0, gb0 = torch.zeros_like(p["k"]), torch.zeros_like(p["bias"])
+        cc.conv_relu_backward_k(p["y"], p["gy"], p["x"], gk0, p["d"])
+        cc.conv_relu_backward_bias(p["y"], p["gy"], gb0)
+        gk1, gb1 = torch.full_like(p["k"], 2.0), torch.full_like(p["bias"], -1.0)   # accumulate semantics
+        cc.conv_relu_backward_kb(p["y"], p["gy"], p["x"], gk1, gb1, p["d"])
+        assert rel_err(gk1 - 2.0, gk0) <= 1e-5
+        assert rel_err(gb1 + 1.0, gb0) <= 1e-5
+
+
+def test_weight_gradient_is_deterministic(cc):
+    p = make_problem(SHAPES_FAST[4], torch.float32, device="cuda")
+    cc.conv_relu_forward(p["x"], p["k"], p["bias"], p["y"], p["d"])
+    runs = []
+    for _ in range(3):
+        gk, gb = torch.zeros_like(p["k"]), torch.zeros_like(p["bias"])
+        cc.conv_relu_backward_kb(p["y"], p["gy"], p["x"], gk, gb, p["d"])
+        runs.append((gk.clone(), gb.clone()))
+    for gk, gb in runs[1:]:
+        assert torch.equal(gk, runs[0][0]) and torch.equal(gb, runs[0][1])
+
+
+def test_output_is_written_in_place_and_constant_input(cc):
+    # ones (*) ones = 9 * C everywhere, borders included (reference tests/test_conv2d.py:47-72)
+    for size, taps in (((20, 33), 9), ((6, 9, 70), 27)):
+        x = torch.ones(1, 3, *size, device="cuda")
+        k = torch.ones(2, 3, *([3] * len(size)), device="cuda")
+        y = torch.empty(1, 2, *size, device="cuda")
+        ptr = y.data_ptr()
+        for d in (1, 2, 5):
+            cc.conv_relu_forward(x, k, torch.zeros(2, device="cuda"), y, d)
+            assert y.data_ptr() == ptr
+            assert torch.equal(y, torch.full_like(y, 3.0 * taps))
+
+
+def test_dilation_error(cc):
+    # reference tests/test_conv2d.py:76-90: 2x2 image, d = 1, 2 fine, d = 3 raises
+    x = torch.zeros(1, 1, 2, 2, device="cuda")
+    k = torch.zeros(1, 1, 3, 3, device="cuda")
+    b = torch.zeros(1, device="cuda")
+    y = torch.zeros(1, 1, 2, 2, device="cuda")
+    cc.conv_forward(x, k, b, y, 1)
+    cc.conv_forward(x, k, b, y, 2)
+    with pytest.raises(RuntimeError):
+        cc.conv_forward(x, k, b, y, 3)
+    with pytest.raises(RuntimeError):
+        cc.conv_relu_forward(x, k, b, y, 0)
+    torch.cuda.synchronize()
+
+
+def test_dtype_and_device_errors(cc):
+    # reference tests/test_conv2d.py:93-106
+    x = torch.zeros(1, 1, 5, 5, device="cuda")
+    k = torch.zeros(1, 1, 3, 3, device="cuda")
+    b = torch.zeros(1, device="cuda")
+    y = torch.zeros(1, 1, 5, 5, device="cuda")
+    with pytest.raises(RuntimeError):
+        cc.conv_forward(x.double(), k, b, y, 1)
+    with pytest.raises(RuntimeError):
+        cc.conv_forward(x.cpu(), k, b, y, 1)
+    with pytest.raises(RuntimeError):
+        cc.conv_relu_forward(x, torch.zeros(1, 1, 3, 6, device="cuda")[..., ::2], b, y, 1)   # non-contiguous kernel
+    with pytest.raises(RuntimeError):
+        cc.conv_relu_forward(x, torch.zeros(1, 2, 3, 3, device="cuda"), b, y, 1)
