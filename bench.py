@@ -1,0 +1,256 @@
+#!/usr/bin/env python3
+"""Headline benchmark: MSD train step (forward + backward) on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C|D|A|B|E2]
+
+Prints ONE JSON line.  `value` is megavoxels per second of one training step
+(batch * voxels / step time) of the workload, inputs resident in HBM.  The
+`roofline` object prices the kernel class that takes the most time against the
+HBM peak using its ALGORITHMIC bytes (every input channel read once per layer,
+the gradient stack read and written once per layer), timed with HIP events on
+the launch stream in an instrumented repeat of the same K steps.  The
+`cpu_baseline` object times the CPU oracle (a C/OpenMP port of the reference
+kernels) on a bounded sample of the same network.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (kind, ndim, c_in, c_out/labels, depth, width, batch, spatial, adam)
+    "A": ("regression", 2, 1, 1, 10, 1, 1, (256, 256), False),
+    "B": ("regression", 2, 1, 1, 100, 1, 4, (512, 512), True),
+    "C": ("segmentation", 2, 1, 4, 100, 1, 1, (1024, 1024), False),
+    "D": ("regression", 3, 1, 1, 50, 1, 1, (128, 128, 128), False),
+    "E2": ("regression", 3, 1, 1, 30, 1, 1, (256, 256, 256), False),
+}
+DESCRIPTION = {
+    "A": "MSDRegressionModel 2D depth 10 width 1, 1x1x256x256, MSE, fwd+bwd",
+    "B": "MSDRegressionModel 2D depth 100 width 1, 4x1x512x512, MSE, fwd+bwd+Adam",
+    "C": "MSDSegmentationModel 2D depth 100 width 1 (4 labels), 1x1x1024x1024, NLL, fwd+bwd",
+    "D": "MSDRegressionModel 3D depth 50 width 1, 1x1x128x128x128, MSE, fwd+bwd",
+    "E2": "MSDRegressionModel 3D depth 30 width 1, 1x1x256x256x256, MSE, fwd+bwd",
+}
+
+
+def make_data(name, torch):
+    kind, ndim, c_in, c_out, depth, width, batch, spatial, adam = WORKLOADS[name]
+    torch.manual_seed(0)
+    if kind == "segmentation":
+        # piecewise-constant blobs (32x32 random labels, nearest-upsampled) + noise
+        grid = torch.randint(0, c_out, (batch, 1, 32, 32))
+        labels = torch.nn.functional.interpolate(grid.float(), size=spatial, mode="nearest").long()
+        x = labels.float() / (c_out - 1) + 0.05 * torch.randn(batch, 1, *spatial)
+        return x, labels
+    x = torch.rand(batch, c_in, *spatial)
+    if name == "B":
+        blur = torch.tensor([[1., 2., 1.], [2., 4., 2.], [1., 2., 1.]]).view(1, 1, 3, 3) / 16
+        return x, torch.nn.functional.conv2d(x, blur, padding=1)
+    return x, x + 0.1 * torch.randn_like(x)
+
+
+def make_model(name, torch):
+    from msd_pytorch_amd import MSDRegressionModel, MSDSegmentationModel
+    kind, ndim, c_in, c_out, depth, width, batch, spatial, adam = WORKLOADS[name]
+    torch.manual_seed(0)
+    if kind == "segmentation":
+        model = MSDSegmentationModel(c_in, c_out, depth, width, ndim=ndim)
+    else:
+        model = MSDRegressionModel(c_in, c_out, depth, width, ndim=ndim)
+    # the final layer starts at zero, which makes every hidden gradient zero
+    # on the first step; give it small random weights so the backward pass
+    # carries real data
+    model.msd.final_layer.linear.weight.data.normal_(0, 0.01)
+    return model
+
+
+def algorithmic_bytes(name):
+    """Per-step algorithmic bytes of each kernel class, fp32:
+    forward (C + w) N 4, backward_x (2C + 2w) N 4, backward_k+bias (C + 2w) N 4,
+    each plus the w*C*K weights."""
+    kind, ndim, c_in, c_out, depth, width, batch, spatial, adam = WORKLOADS[name]
+    n = batch
+    for s in spatial:
+        n *= s
+    K = 3 ** ndim
+    out = {"forward": 0, "backward_x": 0, "backward_kb": 0}
+    for i in range(depth):
+        C = c_in + width * i
+        wts = width * C * K * 4
+        out["forward"] += (C + width) * n * 4 + wts
+        if i > 0:   # layer 0's input gradient is not needed (the network input is data)
+            out["backward_x"] += (2 * C + 2 * width) * n * 4 + wts
+        out["backward_kb"] += (C + 2 * width) * n * 4 + wts
+    return out, n
+
+
+class KernelTimer:
+    """Wraps the operator entry points with HIP events recorded on the current
+    (launch) stream; durations are read after a final synchronise."""
+
+    NAMES = {"conv_relu_forward": "forward", "conv_relu_backward_x": "backward_x",
+             "conv_relu_backward_kb": "backward_kb"}
+
+    def __init__(self, torch, cc):
+        self.torch, self.cc = torch, cc
+        self.events = {v: [] for v in self.NAMES.values()}
+        self.saved = {}
+
+    def __enter__(self):
+        for fn, cls in self.NAMES.items():
+            orig = getattr(self.cc, fn)
+            self.saved[fn] = orig
+
+            def timed(*a, _orig=orig, _cls=cls, **kw):
+                e0 = self.torch.cuda.Event(enable_timing=True)
+                e1 = self.torch.cuda.Event(enable_timing=True)
+                e0.record()
+                _orig(*a, **kw)
+                e1.record()
+                self.events[_cls].append((e0, e1))
+            setattr(self.cc, fn, timed)
+        return self
+
+    def __exit__(self, *exc):
+        for fn, orig in self.saved.items():
+            setattr(self.cc, fn, orig)
+
+    def totals_ms(self):
+        self.torch.cuda.synchronize()
+        return {cls: (sum(a.elapsed_time(b) for a, b in evs), len(evs)) for cls, evs in self.events.items()}
+
+
+def cpu_baseline(name, budget_s=20.0):
+    """Time the CPU oracle's dense-block forward+backward on a bounded sample:
+    the same network on a smaller image, sized from a calibration run."""
+    import torch
+    import oracle
+    kind, ndim, c_in, c_out, depth, width, batch, spatial, adam = WORKLOADS[name]
+    threads = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
+    oracle.set_num_threads(threads)
+    torch.manual_seed(0)
+    dil = [(i % 10) + 1 for i in range(depth)]
+    weights = [torch.randn(width, c_in + width * i, *([3] * ndim)) * (2.0 / (3 ** ndim * (c_in + i))) ** 0.5
+               for i in range(depth)]
+    bias = torch.zeros(depth * width)
+
+    def run(size):
+        x = torch.rand(1, c_in, *size)
+        g = torch.randn(1, c_in + depth * width, *size)
+        t0 = time.perf_counter()
+        res = oracle.block_forward(x, dil, bias, weights)
+        oracle.block_backward(res, g, dil, bias, weights)
+        return time.perf_counter() - t0
+
+    small = (48, 48) if ndim == 2 else (16, 16, 16)
+    t_small = run(small)
+    nv_small = 1
+    for s in small:
+        nv_small *= s
+    # scale the edge so the sample costs about budget_s (cost is linear in voxels)
+    scale = (budget_s / max(t_small, 1e-6)) ** (1.0 / ndim)
+    edge = int(max(small[0], min(small[0] * scale, 384 if ndim == 2 else 48)))
+    size = (edge,) * ndim
+    t = run(size)
+    nv = edge ** ndim
+    return {"value": round(nv / t / 1e6, 4), "unit": "Mvoxel/s", "cores": threads, "kind": "port",
+            "sample": f"C/OpenMP oracle, dense block forward+backward, depth {depth} width {width}, "
+                      f"1x{c_in}x{'x'.join(map(str, size))} fp32, {t:.1f} s"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="C", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-kernel-timing", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU; --gpus must be 1 (no multi-GPU path exists)")
+
+    import torch
+    from msd_pytorch_amd import _native
+    from msd_pytorch_amd import msd_custom_convolutions as cc
+    _native.load()
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+
+    name = args.workload
+    kind, ndim, c_in, c_out, depth, width, batch, spatial, adam = WORKLOADS[name]
+    model = make_model(name, torch)
+    x, target = make_data(name, torch)
+    model.set_input(x)          # inputs resident in HBM before the timed region
+    model.set_target(target)
+
+    def step():
+        model.forward()
+        model.optimizer.zero_grad()
+        model.loss.backward()
+        if adam:
+            model.optimizer.step()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+
+    bytes_per_step, nvox = algorithmic_bytes(name)
+    result = {
+        "metric": "MSD train-step Mvoxel/s",
+        "value": round(nvox / (ms_per_step * 1e-3) / 1e6, 3),
+        "unit": "Mvoxel/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"{name}: {DESCRIPTION[name]}", "depth": depth, "width": width,
+                   "batch": batch, "spatial": list(spatial)},
+    }
+
+    if not args.no_kernel_timing:
+        with KernelTimer(torch, cc) as kt:
+            for _ in range(args.steps):
+                step()
+            totals = kt.totals_ms()
+        kernels = {}
+        for cls, (ms, launches) in totals.items():
+            if launches == 0:
+                continue
+            per_step_ms = ms / args.steps
+            gbs = bytes_per_step[cls] / (per_step_ms * 1e-3) / 1e9
+            kernels[cls] = {"ms_per_step": round(per_step_ms, 4), "launches_per_step": launches // args.steps,
+                            "avg_launch_us": round(ms / launches * 1e3, 2),
+                            "algorithmic_GB_per_step": round(bytes_per_step[cls] / 1e9, 3),
+                            "GBps": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4),
+                            "Mvoxel_per_s": round(nvox / (per_step_ms * 1e-3) / 1e6, 2)}
+        dominant = max(kernels, key=lambda c: kernels[c]["ms_per_step"])
+        result["roofline"] = {"bound": "hbm", "kernel": dominant, "achieved": kernels[dominant]["GBps"],
+                              "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": kernels[dominant]["frac_hbm"],
+                              "traffic": None,
+                              "timed": "HIP events on the launch stream, instrumented repeat of the K steps"}
+        result["kernels"] = kernels
+        hot = sum(k["ms_per_step"] for k in kernels.values())
+        result["hot_path_ms_per_step"] = round(hot, 4)
+
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(name)
+
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
