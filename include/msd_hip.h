@@ -54,6 +54,24 @@ const char *msd_last_error(void);
 int msd_abi_version(void);
 
 /*
+ * Test hook: 0 (default) lets the library pick the specialised gfx950 kernels
+ * where they apply, 1 forces the shape-generic kernels for every call.  Both
+ * paths compute the same operators; the parity tests run each against the other.
+ * Process-wide; not meant to be switched while calls are in flight on other threads.
+ */
+int msd_set_kernel_path(int path);
+
+/*
+ * Tuning hook used by the operator benchmark (the counterpart of the
+ * reference's per-call block_size argument, conv3d.py:8-37): overrides one
+ * launch-shape parameter of the specialised kernels, e.g. "bwdx.vec3d" (voxels
+ * per lane) or "bwdx.unroll3d" (channels in flight).  value < 0 restores the
+ * library default; values a kernel was not built for fall back to the default.
+ * Results do not depend on these settings beyond floating-point summation order.
+ */
+int msd_set_tuning(const char *key, int value);
+
+/*
  * Bytes of device scratch that msd_conv_backward_k, msd_conv_relu_backward_k,
  * msd_conv_relu_backward_kb and msd_conv_relu_backward_bias need for this
  * problem (partial sums of the fixed-order reduction).  Returns < 0 on

@@ -25,6 +25,8 @@ _WS = [_ptr, _c_i64]
 PROTOTYPES = {
     "msd_last_error": (ctypes.c_char_p, []),
     "msd_abi_version": (_c_int, []),
+    "msd_set_kernel_path": (_c_int, [_c_int]),
+    "msd_set_tuning": (_c_int, [ctypes.c_char_p, _c_int]),
     "msd_workspace_bytes": (_c_i64, [_c_int, _c_int, _c_i64, _c_i64, _c_i64, _i64p]),
     "msd_conv_forward": (_c_int, _HEAD + _VIEW + [_ptr, _ptr] + _VIEW + [_ptr]),
     "msd_conv_relu_forward": (_c_int, _HEAD + _VIEW + [_ptr, _ptr] + _VIEW + [_ptr]),

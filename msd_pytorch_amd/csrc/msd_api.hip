@@ -8,9 +8,24 @@
 #include <cstdio>
 #include <string>
 
+namespace msd {
+const char *const kKnobNames[kKnobCount] = {
+    "bwdx.vec2d", "bwdx.vec3d", "bwdx.unroll2d", "bwdx.unroll3d", "bwdx.min_blocks",
+    "xcd_remap",
+};
+int g_knobs[kKnobCount] = {-1, -1, -1, -1, -1, -1};
+int knob(Knob k, int dflt) { return g_knobs[k] < 0 ? dflt : g_knobs[k]; }
+}  // namespace msd
+
 namespace {
 
 thread_local std::string g_error;
+
+// 0: specialised kernels where they apply (default); 1: shape-generic kernels only.
+int g_kernel_path = 0;
+
+template <typename T> struct is_f32 { static constexpr bool value = false; };
+template <> struct is_f32<float> { static constexpr bool value = true; };
 
 int fail(int code, const char *fmt, ...)
 {
@@ -132,7 +147,15 @@ int backward_x_t(const char *fn, bool relu, const msd::Geom &g, int ndim, const 
     MSD_TRY(make_view(fn, "grad_output", ndim, grad_output, gs, &gy));
     MSD_TRY(make_view(fn, "grad_input", ndim, grad_input, xs, &gx));
     if (!kernel) return fail(MSD_ERR_INVALID, "%s: kernel is NULL", fn);
-    hipError_t e = msd::generic_backward_x<T>(g, relu, o, gy, (const T *)kernel, gx, s);
+    hipError_t e;
+    if constexpr (is_f32<T>::value) {
+        if (g_kernel_path == 0 && msd::fast_backward_x_supported(g, relu, o, gy, gx))
+            e = msd::fast_backward_x(g, relu, o, gy, (const float *)kernel, gx, s);
+        else
+            e = msd::generic_backward_x<T>(g, relu, o, gy, (const T *)kernel, gx, s);
+    } else {
+        e = msd::generic_backward_x<T>(g, relu, o, gy, (const T *)kernel, gx, s);
+    }
     return e == hipSuccess ? MSD_OK : hip_fail(fn, e);
 }
 
@@ -186,6 +209,24 @@ extern "C" {
 const char *msd_last_error(void) { return g_error.c_str(); }
 
 int msd_abi_version(void) { return 1; }
+
+int msd_set_tuning(const char *key, int value)
+{
+    if (!key) return fail(MSD_ERR_INVALID, "msd_set_tuning: key is NULL");
+    for (int i = 0; i < msd::kKnobCount; i++)
+        if (std::string(key) == msd::kKnobNames[i]) {
+            msd::g_knobs[i] = value;
+            return MSD_OK;
+        }
+    return fail(MSD_ERR_INVALID, "msd_set_tuning: unknown key '%s'", key);
+}
+
+int msd_set_kernel_path(int path)
+{
+    if (path != 0 && path != 1) return fail(MSD_ERR_INVALID, "msd_set_kernel_path: path must be 0 or 1");
+    g_kernel_path = path;
+    return MSD_OK;
+}
 
 int64_t msd_workspace_bytes(int dtype, int ndim, int64_t batch, int64_t c_in, int64_t c_out, const int64_t *spatial)
 {

@@ -8,6 +8,21 @@ namespace msd {
 
 constexpr int kWave = 64;  // CDNA wavefront width
 
+// MI355X has 8 accelerator dies (XCDs), each with its own L2; workgroups are
+// handed to the XCDs round-robin in launch order.  block_for_xcd() renumbers
+// the workgroups of a grid whose x extent is a multiple of kXcds so that each
+// XCD works on one contiguous range of logical blocks (neighbouring rows and
+// planes, whose halos overlap, then share an L2).  Logical ids >= nblocks are
+// padding and must exit.
+constexpr int kXcds = 8;
+
+inline int xcd_grid(int nblocks) { return (nblocks + kXcds - 1) / kXcds * kXcds; }
+
+__device__ __forceinline__ int block_for_xcd(int bid, int grid, bool remap)
+{
+    return remap ? (bid % kXcds) * (grid / kXcds) + bid / kXcds : bid;
+}
+
 // Problem geometry.  2D problems are carried as D == 1 with NDIM == 2 kernels
 // that have no z taps.
 struct Geom {

@@ -2,6 +2,7 @@
 // double.  One lane per voxel.  These carry the double-precision path and every
 // fp32 problem that the specialised kernels do not accept.
 #include "msd_kernels.h"
+#include "msd_adjoint.h"
 
 namespace msd {
 
@@ -9,15 +10,7 @@ namespace {
 
 constexpr int kBlock = 256;
 
-template <int NDIM> struct Taps { static constexpr int NZ = NDIM == 3 ? 3 : 1; static constexpr int K = NZ * 9; };
 
-__device__ __forceinline__ void decode_voxel(const Geom &g, int n, int &z, int &y, int &x)
-{
-    x = n % g.W;
-    const int t = n / g.W;
-    y = t % g.H;
-    z = t / g.H;
-}
 
 // ---------------------------------------------------------------------------
 // Forward: out = [max(0, .)] (bias + sum_ci sum_taps x[fold(v + dil*tap)] * k)
@@ -76,53 +69,6 @@ __global__ __launch_bounds__(kBlock) void fwd_generic(Geom g, View<const T> x, c
             if (RELU) v = v > T(0) ? v : T(0);
             out.p[o + (int64_t)(co0 + j) * out.sc] = v;
         }
-}
-
-// ---------------------------------------------------------------------------
-// Masked output gradient gathered in adjoint form.  For input voxel u and
-// weight tap t, A[t] = sum of m[v] over all output voxels v whose tap t reads
-// u, with m = grad_output (* [0 < output] when RELU).  Then
-//     grad_input[ci][u]  += sum_t k[co][ci][t] * A[t]            (backward_x)
-//     grad_kernel[co][ci][t] = sum_u x[ci][u] * A[t](u)           (backward_k)
-//     grad_bias[co]          = sum_u A[centre](u)                 (bias)
-// ---------------------------------------------------------------------------
-template <typename T, int NDIM, bool RELU>
-__device__ __forceinline__ void gather_adjoint(const Geom &g, const T *__restrict__ oc, const View<const T> &ov,
-                                               const T *__restrict__ gc, const View<const T> &gv,
-                                               int z, int y, int x, T (&A)[Taps<NDIM>::K])
-{
-    constexpr int NZ = Taps<NDIM>::NZ;
-    const AxisSources sz = NDIM == 3 ? adjoint_sources(z, g.D, g.dil) : single_source();
-    const AxisSources sy = adjoint_sources(y, g.H, g.dil);
-    const AxisSources sx = adjoint_sources(x, g.W, g.dil);
-#pragma unroll
-    for (int p = 0; p < NZ; p++)
-#pragma unroll
-        for (int q = 0; q < 3; q++)
-#pragma unroll
-            for (int r = 0; r < 3; r++) {
-                T s = T(0);
-#pragma unroll
-                for (int a = 0; a < 2; a++) {
-                    if (!sz.ok[p][a]) continue;
-#pragma unroll
-                    for (int bq = 0; bq < 2; bq++) {
-                        if (!sy.ok[q][bq]) continue;
-#pragma unroll
-                        for (int cr = 0; cr < 2; cr++) {
-                            if (!sx.ok[r][cr]) continue;
-                            const int cz = sz.c[p][a], cy = sy.c[q][bq], cx = sx.c[r][cr];
-                            T m = gc[(int64_t)cz * gv.sz + (int64_t)cy * gv.sy + (int64_t)cx * gv.sx];
-                            if (RELU) {
-                                const T o = oc[(int64_t)cz * ov.sz + (int64_t)cy * ov.sy + (int64_t)cx * ov.sx];
-                                m = T(0) < o ? m : T(0);
-                            }
-                            s += m;
-                        }
-                    }
-                }
-                A[(p * 3 + q) * 3 + r] = s;
-            }
 }
 
 // grad_input[b, c0 .. c0+cch) += adjoint; one read-modify-write per output channel.

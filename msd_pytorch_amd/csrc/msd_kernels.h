@@ -25,4 +25,36 @@ template <typename T>
 hipError_t generic_backward_kb(const Geom &g, bool relu, View<const T> out, View<const T> gy, View<const T> x, T *gk,
                                T *gb, T *ws, hipStream_t s);
 
+// Launch-shape knobs (msd_set_tuning in the C ABI).  A value < 0 means "library default".
+enum Knob {
+    kKnobBwdxVec2d, kKnobBwdxVec3d, kKnobBwdxUnroll2d, kKnobBwdxUnroll3d, kKnobBwdxMinBlocks,
+    kKnobXcdRemap,
+    kKnobCount
+};
+int knob(Knob k, int dflt);
+extern const char *const kKnobNames[kKnobCount];
+extern int g_knobs[kKnobCount];
+
+// Specialised fp32 kernels (unit x-stride, one or two output channels).
+bool fast_backward_x_supported_2d(const Geom &g, bool relu, const View<const float> &out,
+                                  const View<const float> &gy, const View<float> &gx);
+bool fast_backward_x_supported_3d(const Geom &g, bool relu, const View<const float> &out,
+                                  const View<const float> &gy, const View<float> &gx);
+hipError_t fast_backward_x_2d(const Geom &g, bool relu, const View<const float> &out, const View<const float> &gy,
+                              const float *k, const View<float> &gx, hipStream_t s);
+hipError_t fast_backward_x_3d(const Geom &g, bool relu, const View<const float> &out, const View<const float> &gy,
+                              const float *k, const View<float> &gx, hipStream_t s);
+
+inline bool fast_backward_x_supported(const Geom &g, bool relu, const View<const float> &out,
+                                      const View<const float> &gy, const View<float> &gx)
+{
+    return g.ndim == 3 ? fast_backward_x_supported_3d(g, relu, out, gy, gx)
+                       : fast_backward_x_supported_2d(g, relu, out, gy, gx);
+}
+inline hipError_t fast_backward_x(const Geom &g, bool relu, const View<const float> &out, const View<const float> &gy,
+                                  const float *k, const View<float> &gx, hipStream_t s)
+{
+    return g.ndim == 3 ? fast_backward_x_3d(g, relu, out, gy, k, gx, s) : fast_backward_x_2d(g, relu, out, gy, k, gx, s);
+}
+
 }  // namespace msd

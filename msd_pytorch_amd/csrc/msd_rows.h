@@ -1,0 +1,176 @@
+// Row-team mapping and LDS-staged adjoint gather shared by the specialised
+// fp32 backward kernels.
+//
+// A workgroup is split into teams of `lpr` lanes; a team owns one image row
+// (z, y) and each lane V consecutive voxels of it.  lpr is a power of two below
+// a wavefront or a multiple of 64, so a wave never holds lanes of a row it
+// shares with another wave only in part.
+//
+// Adjoint gather.  For input voxel u and weight tap t = (p, q, r),
+//     A[t](u) = sum of m(v) over the output voxels v whose tap t reads u,
+// m being the output gradient, masked by [0 < output] when RELU.  Along z and y
+// the sources of a whole row are whole rows (one, or two when the fold of the
+// symmetric padding maps a second row onto it); they are summed while they are
+// staged into LDS:  S[p][q][x] = sum of m over the source rows of (p, q).
+// Along x each voxel then takes at most two values of S per tap (the second
+// again from the fold), read from LDS with clamped indices and select masks, so
+// the code is free of divergent branches.
+//
+// LDS layout of one staged row: element x lives at (x % V) * lpr + x / V, which
+// makes both the V-wide writes and the shifted or mirrored reads of a team hit
+// consecutive banks.
+#pragma once
+
+#include "msd_adjoint.h"
+
+namespace msd {
+
+struct RowTeams {
+    int V;       // voxels per lane
+    int lpr;     // lanes per row
+    int rpw;     // rows (teams) per workgroup
+    int nrows;   // D * H
+};
+
+inline bool make_row_teams(const Geom &g, int V, RowTeams *rt)
+{
+    const int need = (g.W + V - 1) / V;
+    int lpr;
+    if (need <= kWave) {
+        lpr = 1;
+        while (lpr < need) lpr *= 2;
+    } else {
+        lpr = (need + kWave - 1) / kWave * kWave;
+    }
+    if (lpr > 1024) return false;
+    rt->V = V;
+    rt->lpr = lpr;
+    rt->rpw = lpr >= 256 ? 1 : 256 / lpr;
+    rt->nrows = g.D * g.H;
+    return true;
+}
+
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// V consecutive floats as one naturally aligned 4-, 8- or 16-byte access.
+template <int V> __device__ __forceinline__ void load_vec(const float *p, float (&d)[V]);
+template <> __device__ __forceinline__ void load_vec<1>(const float *p, float (&d)[1]) { d[0] = *p; }
+template <> __device__ __forceinline__ void load_vec<2>(const float *p, float (&d)[2])
+{
+    const f32x2 v = *reinterpret_cast<const f32x2 *>(p);
+    d[0] = v[0]; d[1] = v[1];
+}
+template <> __device__ __forceinline__ void load_vec<4>(const float *p, float (&d)[4])
+{
+    const f32x4 v = *reinterpret_cast<const f32x4 *>(p);
+    d[0] = v[0]; d[1] = v[1]; d[2] = v[2]; d[3] = v[3];
+}
+template <int V> __device__ __forceinline__ void store_vec(float *p, const float (&d)[V]);
+template <> __device__ __forceinline__ void store_vec<1>(float *p, const float (&d)[1]) { *p = d[0]; }
+template <> __device__ __forceinline__ void store_vec<2>(float *p, const float (&d)[2])
+{
+    f32x2 v = {d[0], d[1]};
+    *reinterpret_cast<f32x2 *>(p) = v;
+}
+template <> __device__ __forceinline__ void store_vec<4>(float *p, const float (&d)[4])
+{
+    f32x4 v = {d[0], d[1], d[2], d[3]};
+    *reinterpret_cast<f32x4 *>(p) = v;
+}
+
+// True when V-wide accesses at multiples of V along x are naturally aligned
+// for every row of the view.
+template <typename T>
+inline bool rows_aligned(const View<T> &v, int W, int V)
+{
+    if (V == 1) return true;
+    return W % V == 0 && v.sb % V == 0 && v.sc % V == 0 && v.sz % V == 0 && v.sy % V == 0 &&
+           reinterpret_cast<uintptr_t>(v.p) % (V * sizeof(float)) == 0;
+}
+
+template <int NDIM> struct RowTaps { static constexpr int NPQ = NDIM == 3 ? 9 : 3; };
+
+// Floats of LDS one team needs for `wout` output channels.
+template <int NDIM>
+inline size_t staged_floats(const RowTeams &rt, int wout)
+{
+    return (size_t)wout * RowTaps<NDIM>::NPQ * rt.V * rt.lpr;
+}
+
+// Stage S[co][pq] of the team's row into LDS (see the header comment) and keep
+// the lane's own V values of every staged row in `own`.  Every lane of the
+// workgroup must call this; lanes outside the image (`act` false) stage zeros.
+// Ends with a workgroup barrier.
+template <int NDIM, bool RELU, int WOUT, int V>
+__device__ __forceinline__ void stage_source_rows(const Geom &g, const RowTeams &rt, const View<const float> &out,
+                                                  const View<const float> &gy, int b, int z, int y, int lane,
+                                                  bool act, float *__restrict__ S,
+                                                  float (&own)[WOUT][RowTaps<NDIM>::NPQ][V])
+{
+    constexpr int NZ = Taps<NDIM>::NZ;
+    const AxisSources sz = NDIM == 3 ? adjoint_sources(z, g.D, g.dil) : single_source();
+    const AxisSources sy = adjoint_sources(y, g.H, g.dil);
+    const int x0 = lane * V;
+#pragma unroll
+    for (int co = 0; co < WOUT; co++) {
+        const float *gc = gy.p + (int64_t)b * gy.sb + (int64_t)co * gy.sc + x0;
+        const float *oc = RELU ? out.p + (int64_t)b * out.sb + (int64_t)co * out.sc + x0 : nullptr;
+#pragma unroll
+        for (int p = 0; p < NZ; p++)
+#pragma unroll
+            for (int q = 0; q < 3; q++) {
+                float s[V];
+#pragma unroll
+                for (int i = 0; i < V; i++) s[i] = 0.f;
+#pragma unroll
+                for (int a = 0; a < 2; a++)
+#pragma unroll
+                    for (int bq = 0; bq < 2; bq++) {
+                        if (!(act && sz.ok[p][a] && sy.ok[q][bq])) continue;
+                        float m[V];
+                        load_vec<V>(gc + (int64_t)sz.c[p][a] * gy.sz + (int64_t)sy.c[q][bq] * gy.sy, m);
+                        if (RELU) {
+                            float o[V];
+                            load_vec<V>(oc + (int64_t)sz.c[p][a] * out.sz + (int64_t)sy.c[q][bq] * out.sy, o);
+#pragma unroll
+                            for (int i = 0; i < V; i++) m[i] = 0.f < o[i] ? m[i] : 0.f;
+                        }
+#pragma unroll
+                        for (int i = 0; i < V; i++) s[i] += m[i];
+                    }
+                float *row = S + (size_t)(co * RowTaps<NDIM>::NPQ + p * 3 + q) * V * rt.lpr;
+#pragma unroll
+                for (int i = 0; i < V; i++) {
+                    own[co][p * 3 + q][i] = s[i];
+                    row[i * rt.lpr + lane] = s[i];
+                }
+            }
+    }
+    __syncthreads();
+}
+
+// Position of element x in a staged row.
+template <int V>
+__device__ __forceinline__ int staged_index(int x, int lpr)
+{
+    return (x % V) * lpr + x / V;
+}
+
+// The two x-taps that are not the centre, for voxel x of a staged row:
+//   tap 0 (reads x + dil forward):  S[x + dil] if inside,  + S[dil - x - 1]         if x < dil
+//   tap 2 (reads x - dil forward):  S[x - dil] if inside,  + S[2W - x - 1 - dil]    if x + dil >= W
+template <int V>
+__device__ __forceinline__ void side_taps(const float *__restrict__ row, int x, int W, int dil, int lpr, float &t0,
+                                          float &t2)
+{
+    const int hi = x + dil, lo = x - dil;
+    const float a0 = row[staged_index<V>(min(hi, W - 1), lpr)];
+    const float b0 = row[staged_index<V>(max(dil - x - 1, 0), lpr)];
+    const float a2 = row[staged_index<V>(max(lo, 0), lpr)];
+    const float b2 = row[staged_index<V>(min(max(2 * W - x - 1 - dil, 0), W - 1), lpr)];
+    t0 = (hi < W ? a0 : 0.f) + (x < dil ? b0 : 0.f);
+    t2 = (lo >= 0 ? a2 : 0.f) + (hi >= W ? b2 : 0.f);
+}
+
+}  // namespace msd
