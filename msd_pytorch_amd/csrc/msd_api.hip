@@ -11,9 +11,9 @@
 namespace msd {
 const char *const kKnobNames[kKnobCount] = {
     "bwdx.vec2d", "bwdx.vec3d", "bwdx.unroll2d", "bwdx.unroll3d", "bwdx.min_blocks",
-    "xcd_remap",
+    "xcd_remap", "bwdk.vec2d", "bwdk.vec3d", "bwdk.blocks",
 };
-int g_knobs[kKnobCount] = {-1, -1, -1, -1, -1, -1};
+int g_knobs[kKnobCount] = {-1, -1, -1, -1, -1, -1, -1, -1, -1};
 int knob(Knob k, int dflt) { return g_knobs[k] < 0 ? dflt : g_knobs[k]; }
 }  // namespace msd
 
@@ -183,7 +183,15 @@ int backward_kb_t(const char *fn, bool relu, const msd::Geom &g, int ndim, const
     if (grad_kernel) MSD_TRY(make_view(fn, "input", ndim, input, xs, &x));
     if (!grad_kernel && !grad_bias) return fail(MSD_ERR_INVALID, "%s: no gradient buffer given", fn);
     MSD_TRY(check_workspace(fn, g, sizeof(T), ws, ws_bytes));
-    hipError_t e = msd::generic_backward_kb<T>(g, relu, o, gy, x, (T *)grad_kernel, (T *)grad_bias, (T *)ws, s);
+    hipError_t e;
+    if constexpr (is_f32<T>::value) {
+        if (g_kernel_path == 0 && grad_kernel && msd::fast_backward_kb_supported(g, relu, o, gy, x))
+            e = msd::fast_backward_kb(g, relu, o, gy, x, (float *)grad_kernel, (float *)grad_bias, (float *)ws, s);
+        else
+            e = msd::generic_backward_kb<T>(g, relu, o, gy, x, (T *)grad_kernel, (T *)grad_bias, (T *)ws, s);
+    } else {
+        e = msd::generic_backward_kb<T>(g, relu, o, gy, x, (T *)grad_kernel, (T *)grad_bias, (T *)ws, s);
+    }
     return e == hipSuccess ? MSD_OK : hip_fail(fn, e);
 }
 

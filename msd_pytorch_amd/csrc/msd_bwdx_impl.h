@@ -39,16 +39,16 @@ __global__ __launch_bounds__(MAXT) void bwdx_rows(Geom g, RowTeams rt, int cch, 
         float own[WOUT][NPQ][V];
         stage_source_rows<NDIM, RELU, WOUT, V>(g, rt, out, gy, b, z, y, lane, act, S, own);
 #pragma unroll
-        for (int co = 0; co < WOUT; co++)
+        for (int i = 0; i < V; i++) {
+            const SideTaps<V> side(x0 + i, g.W, g.dil, rt.lpr);
 #pragma unroll
-            for (int pq = 0; pq < NPQ; pq++) {
-                const float *srow = S + (size_t)(co * NPQ + pq) * V * rt.lpr;
+            for (int co = 0; co < WOUT; co++)
 #pragma unroll
-                for (int i = 0; i < V; i++) {
-                    side_taps<V>(srow, x0 + i, g.W, g.dil, rt.lpr, A[co][pq * 3 + 0][i], A[co][pq * 3 + 2][i]);
+                for (int pq = 0; pq < NPQ; pq++) {
+                    side.read(S + (size_t)(co * NPQ + pq) * V * rt.lpr, A[co][pq * 3 + 0][i], A[co][pq * 3 + 2][i]);
                     A[co][pq * 3 + 1][i] = own[co][pq][i];
                 }
-            }
+        }
     }
     if (!act) return;
 

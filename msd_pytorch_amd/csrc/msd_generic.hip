@@ -265,7 +265,8 @@ hipError_t launch_bwdk(const Geom &g, View<const T> out, View<const T> gy, View<
 int64_t generic_workspace_elems(const Geom &g)
 {
     const int K = g.ndim == 3 ? 27 : 9;
-    return (int64_t)partial_rows(g) * ((int64_t)g.Wd * g.C * K + g.Wd);
+    // sized for the largest row count any backward_k path uses
+    return (int64_t)kMaxPartialRows * ((int64_t)g.Wd * g.C * K + g.Wd);
 }
 
 template <typename T>

@@ -28,7 +28,7 @@ hipError_t generic_backward_kb(const Geom &g, bool relu, View<const T> out, View
 // Launch-shape knobs (msd_set_tuning in the C ABI).  A value < 0 means "library default".
 enum Knob {
     kKnobBwdxVec2d, kKnobBwdxVec3d, kKnobBwdxUnroll2d, kKnobBwdxUnroll3d, kKnobBwdxMinBlocks,
-    kKnobXcdRemap,
+    kKnobXcdRemap, kKnobBwdkVec2d, kKnobBwdkVec3d, kKnobBwdkBlocks,
     kKnobCount
 };
 int knob(Knob k, int dflt);
@@ -55,6 +55,31 @@ inline hipError_t fast_backward_x(const Geom &g, bool relu, const View<const flo
                                   const float *k, const View<float> &gx, hipStream_t s)
 {
     return g.ndim == 3 ? fast_backward_x_3d(g, relu, out, gy, k, gx, s) : fast_backward_x_2d(g, relu, out, gy, k, gx, s);
+}
+
+// Weight (+ bias) gradient on the matrix cores; gk must not be null, gb may be.
+// ws holds kMaxPartialRows rows of (Wd * C * K + Wd) floats.
+bool fast_backward_kb_supported_2d(const Geom &g, bool relu, const View<const float> &out,
+                                   const View<const float> &gy, const View<const float> &x);
+bool fast_backward_kb_supported_3d(const Geom &g, bool relu, const View<const float> &out,
+                                   const View<const float> &gy, const View<const float> &x);
+hipError_t fast_backward_kb_2d(const Geom &g, bool relu, const View<const float> &out, const View<const float> &gy,
+                               const View<const float> &x, float *gk, float *gb, float *ws, hipStream_t s);
+hipError_t fast_backward_kb_3d(const Geom &g, bool relu, const View<const float> &out, const View<const float> &gy,
+                               const View<const float> &x, float *gk, float *gb, float *ws, hipStream_t s);
+
+inline bool fast_backward_kb_supported(const Geom &g, bool relu, const View<const float> &out,
+                                       const View<const float> &gy, const View<const float> &x)
+{
+    return g.ndim == 3 ? fast_backward_kb_supported_3d(g, relu, out, gy, x)
+                       : fast_backward_kb_supported_2d(g, relu, out, gy, x);
+}
+inline hipError_t fast_backward_kb(const Geom &g, bool relu, const View<const float> &out,
+                                   const View<const float> &gy, const View<const float> &x, float *gk, float *gb,
+                                   float *ws, hipStream_t s)
+{
+    return g.ndim == 3 ? fast_backward_kb_3d(g, relu, out, gy, x, gk, gb, ws, s)
+                       : fast_backward_kb_2d(g, relu, out, gy, x, gk, gb, ws, s);
 }
 
 }  // namespace msd

@@ -108,44 +108,60 @@ __device__ __forceinline__ void stage_source_rows(const Geom &g, const RowTeams 
                                                   bool act, float *__restrict__ S,
                                                   float (&own)[WOUT][RowTaps<NDIM>::NPQ][V])
 {
-    constexpr int NZ = Taps<NDIM>::NZ;
+    constexpr int NZ = Taps<NDIM>::NZ, NPQ = RowTaps<NDIM>::NPQ;
     const AxisSources sz = NDIM == 3 ? adjoint_sources(z, g.D, g.dil) : single_source();
     const AxisSources sy = adjoint_sources(y, g.H, g.dil);
-    const int x0 = lane * V;
+    const int x0 = min(lane * V, g.W - V);   // lanes past the row read a valid address; their values are dropped
+    // rows whose taps fold: within dil of a y (or z) border
+    const bool folds = y < g.dil || y + g.dil >= g.H || (NDIM == 3 && (z < g.dil || z + g.dil >= g.D));
 #pragma unroll
     for (int co = 0; co < WOUT; co++) {
         const float *gc = gy.p + (int64_t)b * gy.sb + (int64_t)co * gy.sc + x0;
         const float *oc = RELU ? out.p + (int64_t)b * out.sb + (int64_t)co * out.sc + x0 : nullptr;
+        float s[NPQ][V];
+        // One masked source row, loaded from a clamped (always valid) address
+        // and zeroed afterwards if it does not count: no branch around the
+        // loads, so all of them are in flight together.
+        auto add_row = [&](int pq, int cz, int cy, bool ok, bool first) {
+            cz = min(max(cz, 0), g.D - 1);
+            cy = min(max(cy, 0), g.H - 1);
+            float m[V];
+            load_vec<V>(gc + (int64_t)cz * gy.sz + (int64_t)cy * gy.sy, m);
+            if (RELU) {
+                float o[V];
+                load_vec<V>(oc + (int64_t)cz * out.sz + (int64_t)cy * out.sy, o);
+#pragma unroll
+                for (int i = 0; i < V; i++) m[i] = 0.f < o[i] ? m[i] : 0.f;
+            }
+#pragma unroll
+            for (int i = 0; i < V; i++) s[pq][i] = (first ? 0.f : s[pq][i]) + (ok && act ? m[i] : 0.f);
+        };
 #pragma unroll
         for (int p = 0; p < NZ; p++)
 #pragma unroll
-            for (int q = 0; q < 3; q++) {
-                float s[V];
+            for (int q = 0; q < 3; q++)
+                add_row(p * 3 + q, sz.c[p][0], sy.c[q][0], sz.ok[p][0] && sy.ok[q][0], true);
+        if (folds) {
 #pragma unroll
-                for (int i = 0; i < V; i++) s[i] = 0.f;
+            for (int p = 0; p < NZ; p++)
 #pragma unroll
-                for (int a = 0; a < 2; a++)
-#pragma unroll
-                    for (int bq = 0; bq < 2; bq++) {
-                        if (!(act && sz.ok[p][a] && sy.ok[q][bq])) continue;
-                        float m[V];
-                        load_vec<V>(gc + (int64_t)sz.c[p][a] * gy.sz + (int64_t)sy.c[q][bq] * gy.sy, m);
-                        if (RELU) {
-                            float o[V];
-                            load_vec<V>(oc + (int64_t)sz.c[p][a] * out.sz + (int64_t)sy.c[q][bq] * out.sy, o);
-#pragma unroll
-                            for (int i = 0; i < V; i++) m[i] = 0.f < o[i] ? m[i] : 0.f;
-                        }
-#pragma unroll
-                        for (int i = 0; i < V; i++) s[i] += m[i];
+                for (int q = 0; q < 3; q++) {
+                    add_row(p * 3 + q, sz.c[p][0], sy.c[q][1], sz.ok[p][0] && sy.ok[q][1], false);
+                    if (NDIM == 3) {
+                        add_row(p * 3 + q, sz.c[p][1], sy.c[q][0], sz.ok[p][1] && sy.ok[q][0], false);
+                        add_row(p * 3 + q, sz.c[p][1], sy.c[q][1], sz.ok[p][1] && sy.ok[q][1], false);
                     }
-                float *row = S + (size_t)(co * RowTaps<NDIM>::NPQ + p * 3 + q) * V * rt.lpr;
-#pragma unroll
-                for (int i = 0; i < V; i++) {
-                    own[co][p * 3 + q][i] = s[i];
-                    row[i * rt.lpr + lane] = s[i];
                 }
+        }
+#pragma unroll
+        for (int pq = 0; pq < NPQ; pq++) {
+            float *row = S + (size_t)(co * NPQ + pq) * V * rt.lpr;
+#pragma unroll
+            for (int i = 0; i < V; i++) {
+                own[co][pq][i] = s[pq][i];
+                row[i * rt.lpr + lane] = s[pq][i];
             }
+        }
     }
     __syncthreads();
 }
@@ -160,17 +176,32 @@ __device__ __forceinline__ int staged_index(int x, int lpr)
 // The two x-taps that are not the centre, for voxel x of a staged row:
 //   tap 0 (reads x + dil forward):  S[x + dil] if inside,  + S[dil - x - 1]         if x < dil
 //   tap 2 (reads x - dil forward):  S[x - dil] if inside,  + S[2W - x - 1 - dil]    if x + dil >= W
+// The four LDS positions and masks depend on x only, so they are computed once
+// per voxel and reused for every staged row.
 template <int V>
-__device__ __forceinline__ void side_taps(const float *__restrict__ row, int x, int W, int dil, int lpr, float &t0,
-                                          float &t2)
-{
-    const int hi = x + dil, lo = x - dil;
-    const float a0 = row[staged_index<V>(min(hi, W - 1), lpr)];
-    const float b0 = row[staged_index<V>(max(dil - x - 1, 0), lpr)];
-    const float a2 = row[staged_index<V>(max(lo, 0), lpr)];
-    const float b2 = row[staged_index<V>(min(max(2 * W - x - 1 - dil, 0), W - 1), lpr)];
-    t0 = (hi < W ? a0 : 0.f) + (x < dil ? b0 : 0.f);
-    t2 = (lo >= 0 ? a2 : 0.f) + (hi >= W ? b2 : 0.f);
-}
+struct SideTaps {
+    int i0a, i0b, i2a, i2b;
+    bool m0a, m0b, m2a, m2b;
+
+    __device__ __forceinline__ SideTaps(int x, int W, int dil, int lpr)
+    {
+        const int hi = x + dil, lo = x - dil;
+        i0a = staged_index<V>(min(hi, W - 1), lpr);
+        i0b = staged_index<V>(max(dil - x - 1, 0), lpr);
+        i2a = staged_index<V>(max(lo, 0), lpr);
+        i2b = staged_index<V>(min(max(2 * W - x - 1 - dil, 0), W - 1), lpr);
+        m0a = hi < W;
+        m0b = x < dil;
+        m2a = lo >= 0;
+        m2b = hi >= W;
+    }
+
+    __device__ __forceinline__ void read(const float *__restrict__ row, float &t0, float &t2) const
+    {
+        const float a0 = row[i0a], b0 = row[i0b], a2 = row[i2a], b2 = row[i2b];
+        t0 = (m0a ? a0 : 0.f) + (m0b ? b0 : 0.f);
+        t2 = (m2a ? a2 : 0.f) + (m2b ? b2 : 0.f);
+    }
+};
 
 }  // namespace msd
