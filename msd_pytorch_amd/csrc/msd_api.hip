@@ -12,8 +12,9 @@ namespace msd {
 const char *const kKnobNames[kKnobCount] = {
     "bwdx.vec2d", "bwdx.vec3d", "bwdx.unroll2d", "bwdx.unroll3d", "bwdx.min_blocks",
     "xcd_remap", "bwdk.vec2d", "bwdk.vec3d", "bwdk.blocks",
+    "fwd.vec2d", "fwd.vec3d", "fwd.split",
 };
-int g_knobs[kKnobCount] = {-1, -1, -1, -1, -1, -1, -1, -1, -1};
+int g_knobs[kKnobCount] = {-1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1};
 int knob(Knob k, int dflt) { return g_knobs[k] < 0 ? dflt : g_knobs[k]; }
 }  // namespace msd
 
@@ -120,7 +121,15 @@ int forward_t(const char *fn, bool relu, const msd::Geom &g, int ndim, const voi
     MSD_TRY(make_view(fn, "output", ndim, output, os, &y));
     if (!kernel) return fail(MSD_ERR_INVALID, "%s: kernel is NULL", fn);
     if (!bias) return fail(MSD_ERR_INVALID, "%s: bias is NULL", fn);
-    hipError_t e = msd::generic_forward<T>(g, relu, x, (const T *)kernel, (const T *)bias, y, s);
+    hipError_t e;
+    if constexpr (is_f32<T>::value) {
+        if (g_kernel_path == 0 && msd::fast_forward_supported(g, x, y))
+            e = msd::fast_forward(g, relu, x, (const float *)kernel, (const float *)bias, y, s);
+        else
+            e = msd::generic_forward<T>(g, relu, x, (const T *)kernel, (const T *)bias, y, s);
+    } else {
+        e = msd::generic_forward<T>(g, relu, x, (const T *)kernel, (const T *)bias, y, s);
+    }
     return e == hipSuccess ? MSD_OK : hip_fail(fn, e);
 }
 

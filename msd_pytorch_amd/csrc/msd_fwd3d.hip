@@ -1,0 +1,17 @@
+// forward, 3D instantiations (one file per rank so they compile in parallel).
+#include "msd_fwd_impl.h"
+
+namespace msd {
+
+bool fast_forward_supported_3d(const Geom &g, const View<const float> &x, const View<float> &out)
+{
+    return fwd::supported_nd<3>(g, x, out);
+}
+
+hipError_t fast_forward_3d(const Geom &g, bool relu, const View<const float> &x, const float *k, const float *bias,
+                            const View<float> &out, hipStream_t s)
+{
+    return fwd::run_nd<3>(g, relu, x, k, bias, out, s);
+}
+
+}  // namespace msd

@@ -1,0 +1,259 @@
+// Forward pass for fp32 with unit x-stride and one or two output channels:
+//     out[v] = [max(0, .)] ( bias + sum_ci sum_{p,q,r} x[ci][fold(v + dil*(p,q,r))] * k[ci][p][q][r] )
+//
+// Work split.  A team of `lpr` lanes (a multiple of 64) owns full image rows,
+// V consecutive voxels per lane.  One workgroup computes a small lattice of
+// RZ x RY output rows whose members are dil apart in z and y:
+//     rows (z0 + jz*dil, y0 + jy*dil),  jz < RZ, jy < RY.
+// Their 3x3 (x3) taps fall on the (RZ+2) x (RY+2) input rows of the same
+// lattice, so each input row that is loaded serves up to nine output rows from
+// registers (an ordinary square tile would need a halo of 2*dil rows).
+// Along x nothing is shifted in the channel loop at all: for every output row
+// the lane accumulates the three partial sums
+//     T_r[x'] = sum_ci sum_{p,q} x[ci][..][x'] * k[ci][p][q][r],      r = 0, 1, 2
+// at its own positions x', and the row is finished once, after the channel
+// loop, as  out[x] = T_0[fold(x - dil)] + T_1[x] + T_2[fold(x + dil)]  through LDS.
+// The channel loop is therefore: one aligned V-wide load per input row, then
+// 3*V fused multiply-adds per (output row, tap row) pair, with wave-uniform
+// weights from scalar registers.
+//
+// The input channels are split over KS groups of lanes of the workgroup
+// (channel ci goes to group ci % KS), which multiplies the number of waves in
+// flight; the groups' partial sums meet in LDS in the finishing step, in a fixed order.
+// Algorithmic traffic: (C + w) * N * 4 bytes.
+#pragma once
+#include "msd_kernels.h"
+#include "msd_rows.h"
+
+namespace msd {
+namespace fwd {
+
+struct Lattice {
+    int lpr;        // lanes per row
+    int ks;         // channel groups per workgroup
+    int segs_y;     // lattice segments per y residue
+    int segs_z;
+    int tiles_y;    // dil * segs_y
+    int tiles_z;    // dil * segs_z (1 in 2D)
+    int ntiles;
+};
+
+template <int NDIM, bool RELU, int WOUT, int V, int RZ, int RY>
+__global__ __launch_bounds__(1024) void fwd_lattice(Geom g, Lattice lt, int remap, View<const float> x,
+                                                    const float *__restrict__ k, const float *__restrict__ bias,
+                                                    View<float> out)
+{
+    extern __shared__ float lds[];
+    constexpr int K = Taps<NDIM>::K;
+    constexpr int NZ = Taps<NDIM>::NZ;          // z taps: 3 or 1
+    constexpr int LZ = NDIM == 3 ? RZ + 2 : 1;  // input lattice levels along z
+    constexpr int LY = RY + 2;
+    static_assert(NDIM == 3 || RZ == 1, "2D has a single z level");
+
+    const int tile = block_for_xcd(blockIdx.x, gridDim.x, remap);
+    if (tile >= lt.ntiles) return;               // padding block
+    const int ty = tile % lt.tiles_y, tz = tile / lt.tiles_y;
+    const int y0 = ty / lt.segs_y + (ty % lt.segs_y) * RY * g.dil;
+    const int z0 = NDIM == 3 ? tz / lt.segs_z + (tz % lt.segs_z) * RZ * g.dil : 0;
+    if (y0 >= g.H || z0 >= g.D) return;          // empty tail of a residue class (whole workgroup)
+
+    const int lane = threadIdx.x % lt.lpr;
+    const int kg = __builtin_amdgcn_readfirstlane(threadIdx.x / lt.lpr);   // uniform: lpr is a multiple of 64
+    const int x0 = min(lane * V, g.W - V);       // lanes past the row load a valid address; nothing is stored
+    const bool act = lane * V < g.W;
+    const int b = blockIdx.y;
+
+    // element offsets of the input lattice rows (fold, then clamp rows that only
+    // feed output rows outside the image)
+    int64_t offz[LZ], offy[LY];
+#pragma unroll
+    for (int m = 0; m < LZ; m++)
+        offz[m] = NDIM == 3 ? (int64_t)min(reflect_idx(min(z0 + (m - 1) * g.dil, 2 * g.D - 1), g.D), g.D - 1) * x.sz : 0;
+#pragma unroll
+    for (int m = 0; m < LY; m++)
+        offy[m] = (int64_t)min(reflect_idx(min(y0 + (m - 1) * g.dil, 2 * g.H - 1), g.H), g.H - 1) * x.sy;
+
+    float acc[WOUT][RZ][RY][3][V];
+#pragma unroll
+    for (int co = 0; co < WOUT; co++)
+#pragma unroll
+        for (int jz = 0; jz < RZ; jz++)
+#pragma unroll
+            for (int jy = 0; jy < RY; jy++)
+#pragma unroll
+                for (int r = 0; r < 3; r++)
+#pragma unroll
+                    for (int i = 0; i < V; i++) acc[co][jz][jy][r][i] = 0.f;
+
+    const float *xb = x.p + (int64_t)b * x.sb + x0;
+    for (int ci = kg; ci < g.C; ci += lt.ks) {
+        const float *xc = xb + (int64_t)ci * x.sc;
+        float w[WOUT][K];
+#pragma unroll
+        for (int co = 0; co < WOUT; co++)
+#pragma unroll
+            for (int t = 0; t < K; t++) w[co][t] = k[((int64_t)co * g.C + ci) * K + t];
+#pragma unroll
+        for (int mz = 0; mz < LZ; mz++)
+#pragma unroll
+            for (int my = 0; my < LY; my++) {
+                float xv[V];
+                load_vec<V>(xc + offz[mz] + offy[my], xv);
+#pragma unroll
+                for (int p = 0; p < NZ; p++) {
+                    const int jz = NDIM == 3 ? mz - p : 0;       // input level m = j + p  (p, q counted from 0)
+                    if (jz < 0 || jz >= RZ) continue;
+#pragma unroll
+                    for (int q = 0; q < 3; q++) {
+                        const int jy = my - q;
+                        if (jy < 0 || jy >= RY) continue;
+#pragma unroll
+                        for (int co = 0; co < WOUT; co++)
+#pragma unroll
+                            for (int r = 0; r < 3; r++) {
+                                const float wv = w[co][(p * 3 + q) * 3 + r];
+#pragma unroll
+                                for (int i = 0; i < V; i++) acc[co][jz][jy][r][i] += xv[i] * wv;
+                            }
+                    }
+                }
+            }
+    }
+
+    // Finish the rows one at a time.  LDS holds T_r of the current row for every
+    // channel group: T[kg][r][staged x]; group (row counter % KS) adds the groups
+    // up at the three shifted positions and writes the row.
+    const int rowlen = V * lt.lpr;
+    float *T = lds;
+    int counter = 0;
+#pragma unroll
+    for (int co = 0; co < WOUT; co++) {
+        const float bv = bias[co];
+#pragma unroll
+        for (int jz = 0; jz < RZ; jz++)
+#pragma unroll
+            for (int jy = 0; jy < RY; jy++) {
+                const int z = z0 + jz * g.dil, y = y0 + jy * g.dil;
+                if (z >= g.D || y >= g.H) continue;             // uniform over the workgroup
+#pragma unroll
+                for (int r = 0; r < 3; r++)
+#pragma unroll
+                    for (int i = 0; i < V; i++)
+                        T[(kg * 3 + r) * rowlen + i * lt.lpr + lane] = act ? acc[co][jz][jy][r][i] : 0.f;
+                __syncthreads();
+                if (kg == counter % lt.ks && act) {
+                    float o[V];
+#pragma unroll
+                    for (int i = 0; i < V; i++) {
+                        const int xx = x0 + i;
+                        const int i0 = staged_index<V>(reflect_idx(xx - g.dil, g.W), lt.lpr);
+                        const int i1 = i * lt.lpr + lane;
+                        const int i2 = staged_index<V>(reflect_idx(xx + g.dil, g.W), lt.lpr);
+                        float s = bv;
+                        for (int kk = 0; kk < lt.ks; kk++) {
+                            const float *tk = T + (size_t)kk * 3 * rowlen;
+                            s += tk[i0] + tk[rowlen + i1] + tk[2 * rowlen + i2];
+                        }
+                        o[i] = RELU ? (s > 0.f ? s : 0.f) : s;
+                    }
+                    store_vec<V>(out.p + (int64_t)b * out.sb + (int64_t)co * out.sc + (int64_t)z * out.sz +
+                                     (int64_t)y * out.sy + x0,
+                                 o);
+                }
+                counter++;
+                __syncthreads();
+            }
+    }
+}
+
+constexpr size_t kMaxLds = 64 * 1024;
+
+inline bool make_lattice(const Geom &g, int V, int rz, int ry, int ks_wanted, Lattice *lt)
+{
+    const int need = (g.W + V - 1) / V;
+    const int lpr = (need + kWave - 1) / kWave * kWave;
+    if (lpr > 1024) return false;
+    int ks = ks_wanted;
+    while (ks > 1 && (ks * lpr > 1024 || ks > g.C)) ks /= 2;
+    if ((size_t)ks * 3 * V * lpr * sizeof(float) > kMaxLds) return false;
+    lt->lpr = lpr;
+    lt->ks = ks;
+    lt->segs_y = ((g.H + g.dil - 1) / g.dil + ry - 1) / ry;
+    lt->tiles_y = g.dil * lt->segs_y;
+    if (g.ndim == 3) {
+        lt->segs_z = ((g.D + g.dil - 1) / g.dil + rz - 1) / rz;
+        lt->tiles_z = g.dil * lt->segs_z;
+    } else {
+        lt->segs_z = 1;
+        lt->tiles_z = 1;
+    }
+    lt->ntiles = lt->tiles_y * lt->tiles_z;
+    return true;
+}
+
+template <int NDIM, bool RELU, int WOUT, int V, int RZ, int RY>
+hipError_t launch(const Geom &g, const View<const float> &x, const float *k, const float *bias,
+                  const View<float> &out, hipStream_t s)
+{
+    Lattice lt;
+    if (!make_lattice(g, V, RZ, RY, knob(kKnobFwdSplit, NDIM == 3 ? 4 : 2), &lt)) return hipErrorInvalidConfiguration;
+    const int remap = knob(kKnobXcdRemap, 1);
+    const dim3 grid(remap ? xcd_grid(lt.ntiles) : lt.ntiles, g.B, 1);
+    const size_t lds = (size_t)lt.ks * 3 * V * lt.lpr * sizeof(float);
+    hipLaunchKernelGGL((fwd_lattice<NDIM, RELU, WOUT, V, RZ, RY>), grid, dim3(lt.ks * lt.lpr), lds, s, g, lt, remap, x,
+                       k, bias, out);
+    return hipGetLastError();
+}
+
+// Largest V whose accesses are aligned in both views and that leaves at least
+// one full wave per row.
+inline int choose_vec(const Geom &g, int vmax, const View<const float> &x, const View<float> &out)
+{
+    for (int v = 4; v >= 1; v /= 2) {
+        if (v > vmax) continue;
+        if (!rows_aligned(x, g.W, v) || !rows_aligned(out, g.W, v)) continue;
+        if (v > 1 && (g.W + v - 1) / v < kWave) continue;   // keep the lanes of a wave busy
+        if ((g.W + v - 1) / v > 1024) continue;
+        return v;
+    }
+    return 0;
+}
+
+template <int NDIM>
+bool supported_nd(const Geom &g, const View<const float> &x, const View<float> &out)
+{
+    if (g.Wd > 2 || x.sx != 1 || out.sx != 1) return false;
+    if (g.W < 32) return false;                  // rows shorter than half a wave: the generic kernel does better
+    return choose_vec(g, 4, x, out) != 0;
+}
+
+template <int NDIM, bool RELU, int WOUT>
+hipError_t pick(const Geom &g, const View<const float> &x, const float *k, const float *bias, const View<float> &out,
+                hipStream_t s)
+{
+    const int vmax = knob(NDIM == 3 ? kKnobFwdVec3d : kKnobFwdVec2d, NDIM == 3 ? 1 : 4);
+    int v = choose_vec(g, vmax, x, out);
+    if (v == 0) v = choose_vec(g, 4, x, out);
+    if constexpr (NDIM == 3) {
+        if (v == 4) return launch<3, RELU, WOUT, 4, 2, 2>(g, x, k, bias, out, s);
+        if (v == 2) return launch<3, RELU, WOUT, 2, 2, 4>(g, x, k, bias, out, s);
+        if (v == 1) return launch<3, RELU, WOUT, 1, 2, 4>(g, x, k, bias, out, s);
+    } else {
+        if (v == 4) return launch<2, RELU, WOUT, 4, 1, 4>(g, x, k, bias, out, s);
+        if (v == 2) return launch<2, RELU, WOUT, 2, 1, 4>(g, x, k, bias, out, s);
+        if (v == 1) return launch<2, RELU, WOUT, 1, 1, 4>(g, x, k, bias, out, s);
+    }
+    return hipErrorInvalidConfiguration;
+}
+
+template <int NDIM>
+hipError_t run_nd(const Geom &g, bool relu, const View<const float> &x, const float *k, const float *bias,
+                  const View<float> &out, hipStream_t s)
+{
+    if (g.Wd == 1)
+        return relu ? pick<NDIM, true, 1>(g, x, k, bias, out, s) : pick<NDIM, false, 1>(g, x, k, bias, out, s);
+    return relu ? pick<NDIM, true, 2>(g, x, k, bias, out, s) : pick<NDIM, false, 2>(g, x, k, bias, out, s);
+}
+
+}  // namespace fwd
+}  // namespace msd

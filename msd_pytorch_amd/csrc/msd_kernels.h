@@ -29,6 +29,7 @@ hipError_t generic_backward_kb(const Geom &g, bool relu, View<const T> out, View
 enum Knob {
     kKnobBwdxVec2d, kKnobBwdxVec3d, kKnobBwdxUnroll2d, kKnobBwdxUnroll3d, kKnobBwdxMinBlocks,
     kKnobXcdRemap, kKnobBwdkVec2d, kKnobBwdkVec3d, kKnobBwdkBlocks,
+    kKnobFwdVec2d, kKnobFwdVec3d, kKnobFwdSplit,
     kKnobCount
 };
 int knob(Knob k, int dflt);
@@ -55,6 +56,23 @@ inline hipError_t fast_backward_x(const Geom &g, bool relu, const View<const flo
                                   const float *k, const View<float> &gx, hipStream_t s)
 {
     return g.ndim == 3 ? fast_backward_x_3d(g, relu, out, gy, k, gx, s) : fast_backward_x_2d(g, relu, out, gy, k, gx, s);
+}
+
+bool fast_forward_supported_2d(const Geom &g, const View<const float> &x, const View<float> &out);
+bool fast_forward_supported_3d(const Geom &g, const View<const float> &x, const View<float> &out);
+hipError_t fast_forward_2d(const Geom &g, bool relu, const View<const float> &x, const float *k, const float *bias,
+                           const View<float> &out, hipStream_t s);
+hipError_t fast_forward_3d(const Geom &g, bool relu, const View<const float> &x, const float *k, const float *bias,
+                           const View<float> &out, hipStream_t s);
+
+inline bool fast_forward_supported(const Geom &g, const View<const float> &x, const View<float> &out)
+{
+    return g.ndim == 3 ? fast_forward_supported_3d(g, x, out) : fast_forward_supported_2d(g, x, out);
+}
+inline hipError_t fast_forward(const Geom &g, bool relu, const View<const float> &x, const float *k,
+                               const float *bias, const View<float> &out, hipStream_t s)
+{
+    return g.ndim == 3 ? fast_forward_3d(g, relu, x, k, bias, out, s) : fast_forward_2d(g, relu, x, k, bias, out, s);
 }
 
 // Weight (+ bias) gradient on the matrix cores; gk must not be null, gb may be.
