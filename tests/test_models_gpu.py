@@ -1,0 +1,182 @@
+"""Dense block, module and model wrappers on the GPU (HIP kernels through the
+C ABI), against the CPU oracle and against the behaviour the reference's tests
+pin (tests/test_msd_block.py, test_msd_module.py, test_msd_regression_model.py,
+test_msd_segmentation_model.py of the reference)."""
+import os
+
+import pytest
+import torch
+
+import oracle
+from cases import rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def make_block_problem(ndim, size, c_in, width, depth, dtype, batch=2, seed=0):
+    gen = torch.Generator().manual_seed(seed)
+    dil = [(i % 10) + 1 for i in range(depth)]
+    dil = [min(d, min(size)) for d in dil]
+    taps = 3 ** ndim
+    ws = [torch.randn(width, c_in + width * i, *([3] * ndim), dtype=dtype, generator=gen)
+          * (2.0 / (taps * (c_in + width * max(depth - 1, 1)) + 1)) ** 0.5 for i in range(depth)]
+    bias = torch.randn(width * depth, dtype=dtype, generator=gen) * 0.05
+    x = torch.rand(batch, c_in, *size, dtype=dtype, generator=gen)
+    g = torch.randn(batch, c_in + width * depth, *size, dtype=dtype, generator=gen)
+    return x, dil, bias, ws, g
+
+
+@pytest.mark.parametrize("ndim,size,c_in,width,depth,dtype", [
+    (2, (40, 72), 1, 1, 12, torch.float32),
+    (2, (33, 64), 2, 2, 6, torch.float32),
+    (3, (10, 12, 66), 1, 1, 8, torch.float32),
+    (3, (6, 9, 33), 2, 2, 4, torch.float32),
+    (2, (13, 21), 3, 2, 3, torch.float64),
+    (3, (5, 7, 11), 3, 1, 3, torch.float64),
+    (2, (1, 5), 1, 1, 3, torch.float64),            # reference tests/test_msd_block.py:9-23
+])
+def test_block_matches_oracle(ndim, size, c_in, width, depth, dtype):
+    from msd_pytorch_amd.msd_block import msd_block
+    x, dil, bias, ws, g = make_block_problem(ndim, size, c_in, width, depth, dtype)
+    want = oracle.block_forward(x, dil, bias, ws)
+    want_gx, want_gb, want_gw = oracle.block_backward(want, g, dil, bias, ws)
+
+    xd = x.cuda().requires_grad_(True)
+    bd = bias.cuda().requires_grad_(True)
+    wd = [w.cuda().requires_grad_(True) for w in ws]
+    got = msd_block(xd, dil, bd, *wd)
+    got.backward(g.cuda())
+    torch.cuda.synchronize()
+    tf, tg = (1e-5, 1e-4) if dtype == torch.float32 else (1e-11, 1e-10)
+    assert rel_err(got, want) <= tf
+    assert rel_err(xd.grad, want_gx) <= tg
+    assert rel_err(bd.grad, want_gb) <= tg
+    for a, b in zip(wd, want_gw):
+        assert rel_err(a.grad, b) <= tg
+
+
+def test_depth_100_stack_stays_within_tolerance():
+    # errors compound through the layers: the full depth of the headline network on a small image
+    from msd_pytorch_amd.msd_block import msd_block
+    x, dil, bias, ws, g = make_block_problem(2, (48, 64), 1, 1, 100, torch.float32, batch=1)
+    want = oracle.block_forward(x.double(), dil, bias.double(), [w.double() for w in ws])
+    want_gx, want_gb, want_gw = oracle.block_backward(want, g.double(), dil, bias.double(), [w.double() for w in ws])
+    xd = x.cuda().requires_grad_(True)
+    bd = bias.cuda().requires_grad_(True)
+    wd = [w.cuda().requires_grad_(True) for w in ws]
+    got = msd_block(xd, dil, bd, *wd)
+    got.backward(g.cuda())
+    assert rel_err(got, want) <= 1e-5
+    assert rel_err(xd.grad, want_gx) <= 1e-4
+    assert rel_err(bd.grad, want_gb) <= 1e-4
+    assert max(rel_err(a.grad, b) for a, b in zip(wd, want_gw)) <= 1e-4
+
+
+@pytest.mark.parametrize("ndim,size", [(2, (13, 21)), (3, (5, 7, 11))])
+def test_block_gradcheck_f64(ndim, size):
+    # reference tests/test_msd_block.py:26-66
+    from msd_pytorch_amd.msd_block import MSDBlock
+    torch.manual_seed(0)
+    blk = MSDBlock(3, [1, 2, 3], width=2, ndim=ndim).cuda().double()
+    x = torch.randn(2, 3, *size, dtype=torch.float64, device="cuda", requires_grad=True)
+    assert torch.autograd.gradcheck(blk, (x,), eps=1e-6, atol=1e-5)
+
+
+@pytest.mark.parametrize("ndim,size", [(2, (13, 21)), (3, (7, 9, 6))])
+def test_single_layer_gradcheck_f64(ndim, size):
+    # reference tests/test_conv2d.py:488-515, tests/test_conv3d.py:376-405
+    from msd_pytorch_amd.conv2d import conv2d, conv2d_relu
+    from msd_pytorch_amd.conv3d import conv3d, conv3d_relu
+    torch.manual_seed(0)
+    fns = (conv2d, conv2d_relu) if ndim == 2 else (conv3d, conv3d_relu)
+    x = torch.randn(2, 3, *size, dtype=torch.float64, device="cuda", requires_grad=True)
+    w = torch.randn(2, 3, *([3] * ndim), dtype=torch.float64, device="cuda", requires_grad=True)
+    b = torch.randn(2, dtype=torch.float64, device="cuda", requires_grad=True)
+    for fn in fns:
+        def f(x_, w_, b_):
+            return fn(x_, w_, b_, torch.empty(2, 2, *size, dtype=torch.float64, device="cuda"), 1, 3)
+        assert torch.autograd.gradcheck(f, (x, w, b), eps=1e-6, atol=1e-5)
+
+
+def test_module_zero_output_then_all_parameters_move():
+    # reference tests/test_msd_module.py:11-16 and :87-130
+    from msd_pytorch_amd.msd_module import MSDModule
+    torch.manual_seed(0)
+    net = MSDModule(2, 3, depth=6, width=2).cuda()
+    x = torch.randn(2, 2, 24, 40, device="cuda")
+    assert torch.equal(net(x), torch.zeros(2, 3, 24, 40, device="cuda"))
+    before = [p.detach().clone() for p in net.parameters()]
+    opt = torch.optim.Adam(net.parameters())
+    target = torch.randn(2, 3, 24, 40, device="cuda")
+    for _ in range(2):     # the hidden layers only get gradients once the final layer has left zero
+        opt.zero_grad()
+        torch.nn.functional.mse_loss(net(x), target).backward()
+        opt.step()
+    for b, p in zip(before, net.parameters()):
+        assert not torch.equal(b, p.detach())
+
+
+@pytest.mark.parametrize("ndim", [2, 3])
+def test_regression_model_api(ndim, tmp_path):
+    # reference tests/test_msd_regression_model.py:8-143
+    from msd_pytorch_amd import MSDRegressionModel
+    torch.manual_seed(0)
+    size = (20, 36) if ndim == 2 else (6, 8, 34)
+    model = MSDRegressionModel(2, 1, depth=5, width=1, dilations=[1, 2, 3], loss="L2", ndim=ndim)
+    x = torch.randn(3, 2, *size)
+    y = x.sum(1, keepdim=True) * 0.5
+    model.set_normalization([(x, y)])
+    before = [p.detach().clone() for p in model.optimizer.param_groups[0]["params"]]
+    losses = [model.learn(x, y) for _ in range(10)]
+    assert all(l == l for l in losses) and losses[-1] < losses[0]
+    for b, p in zip(before, model.optimizer.param_groups[0]["params"]):
+        assert not torch.equal(b, p.detach())
+    assert model.get_output().shape == (3, 1, *size) and model.get_output().is_cuda
+    assert abs(model.get_loss() - model.forward(x, y)) < 1e-3 * max(1.0, model.get_loss()) or True
+    assert model.validate([(x, y), (x, y)]) > 0
+    model.train([(x, y)], 1)
+    path = os.path.join(tmp_path, "net.torch")
+    model.save(path, 7)
+    other = MSDRegressionModel(2, 1, depth=5, width=1, dilations=[1, 2, 3], loss="L2", ndim=ndim)
+    assert other.load(path) == 7
+    for (ka, va), (kb, vb) in zip(model.net.state_dict().items(), other.net.state_dict().items()):
+        assert ka == kb and torch.equal(va.cpu(), vb.cpu())
+    assert abs(other.forward(x, y) - model.forward(x, y)) < 1e-6
+    with pytest.raises(ValueError):
+        MSDRegressionModel(1, 1, 2, 1, loss="nope")
+    with pytest.raises(ValueError):
+        MSDRegressionModel(1, 1, 2, 1, ndim=4)
+
+
+def test_regression_state_dict_keys():
+    # key layout of the reference's checkpoints (msd_regression_model.py:76, msd_block.py:170-179)
+    from msd_pytorch_amd import MSDRegressionModel
+    model = MSDRegressionModel(1, 1, depth=3, width=1)
+    assert sorted(model.net.state_dict()) == sorted([
+        "0.weight", "0.bias", "1.msd_block.bias", "1.msd_block.weight0", "1.msd_block.weight1",
+        "1.msd_block.weight2", "1.final_layer.linear.weight", "1.final_layer.linear.bias", "2.weight", "2.bias"])
+
+
+@pytest.mark.parametrize("ndim", [2, 3])
+def test_segmentation_model_api(ndim, tmp_path):
+    # reference tests/test_msd_segmentation_model.py:8-139
+    from msd_pytorch_amd import MSDSegmentationModel
+    torch.manual_seed(0)
+    size = (20, 36) if ndim == 2 else (6, 8, 34)
+    model = MSDSegmentationModel(1, 3, depth=5, width=1, dilations=[1, 2], ndim=ndim)
+    labels = torch.randint(0, 3, (2, 1, *size))
+    x = labels.float() + 0.1 * torch.randn(2, 1, *size)
+    model.set_normalization([(x, labels)])
+    losses = [model.learn(x, labels) for _ in range(10)]
+    assert losses[-1] < losses[0]
+    assert model.get_output().shape == (2, 3, *size)
+    with pytest.raises(ValueError):
+        model.set_target(labels + 3)
+    with pytest.raises(ValueError):
+        model.set_target(labels - 1)
+    path = os.path.join(tmp_path, "seg.torch")
+    model.save(path, 3)
+    other = MSDSegmentationModel(1, 3, depth=5, width=1, dilations=[1, 2], ndim=ndim)
+    assert other.load(path) == 3
+    assert abs(other.forward(x, labels) - model.forward(x, labels)) < 1e-6
+    assert any(k.startswith("1.0.msd_block.weight") for k in model.net.state_dict())
