@@ -173,6 +173,8 @@ def main():
     ap.add_argument("--workload", default="C", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-timing", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run one 1 GiB device copy first (reference dispatch for scaling rocprof byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; --gpus must be 1 (no multi-GPU path exists)")
@@ -183,6 +185,13 @@ def main():
     _native.load()
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
+
+    if args.calibrate_copy:
+        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)          # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
 
     name = args.workload
     kind, ndim, c_in, c_out, depth, width, batch, spatial, adam = WORKLOADS[name]
