@@ -95,8 +95,11 @@ class KernelTimer:
     """Wraps the operator entry points with HIP events recorded on the current
     (launch) stream; durations are read after a final synchronise."""
 
-    NAMES = {"conv_relu_forward": "forward", "conv_relu_backward_x": "backward_x",
-             "conv_relu_backward_kb": "backward_kb"}
+    # the dense block applies the ReLU mask to its gradient stack once per layer
+    # (relu_mask_gradient, timed with backward_x, whose on-the-fly mask it replaces)
+    # and then calls the plain backward operators
+    NAMES = {"conv_relu_forward": "forward", "relu_mask_gradient": "backward_x", "conv_backward_x": "backward_x",
+             "conv_backward_kb": "backward_kb"}
 
     def __init__(self, torch, cc):
         self.torch, self.cc = torch, cc
@@ -241,8 +244,8 @@ def main():
                 continue
             per_step_ms = ms / args.steps
             gbs = bytes_per_step[cls] / (per_step_ms * 1e-3) / 1e9
-            kernels[cls] = {"ms_per_step": round(per_step_ms, 4), "launches_per_step": launches // args.steps,
-                            "avg_launch_us": round(ms / launches * 1e3, 2),
+            kernels[cls] = {"ms_per_step": round(per_step_ms, 4), "calls_per_step": launches // args.steps,
+                            "avg_call_us": round(ms / launches * 1e3, 2),
                             "algorithmic_GB_per_step": round(bytes_per_step[cls] / 1e9, 3),
                             "GBps": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4),
                             "Mvoxel_per_s": round(nvox / (per_step_ms * 1e-3) / 1e6, 2)}

@@ -166,6 +166,24 @@ int msd_conv_relu_backward_kb(int dtype, int ndim, int64_t batch, int64_t c_in, 
                               void *grad_kernel, void *grad_bias,
                               void *workspace, int64_t workspace_bytes, void *stream);
 
+/* msd_conv_backward_k and msd_conv_backward_bias in one pass (no ReLU mask).
+ * grad_bias may be NULL.  No counterpart in the reference. */
+int msd_conv_backward_kb(int dtype, int ndim, int64_t batch, int64_t c_in, int64_t c_out,
+                         const int64_t *spatial, int dilation,
+                         const void *grad_output, const int64_t *grad_output_strides,
+                         const void *input, const int64_t *input_strides,
+                         void *grad_kernel, void *grad_bias,
+                         void *workspace, int64_t workspace_bytes, void *stream);
+
+/* grad_output = grad_output * [0 < output], in place: the ReLU mask that the three
+ * conv_relu_backward_* operators of one layer (msd_block.py:107-126) each apply on
+ * the fly, applied once.  After it the plain backward operators give the layer's
+ * gradients.  Only valid when the caller owns grad_output and no longer needs the
+ * unmasked values, as in the dense block's private gradient stack (msd_block.py:83). */
+int msd_relu_mask_gradient(int dtype, int ndim, int64_t batch, int64_t c_out, const int64_t *spatial,
+                           const void *output, const int64_t *output_strides,
+                           void *grad_output, const int64_t *grad_output_strides, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -38,6 +38,8 @@ PROTOTYPES = {
     "msd_conv_relu_backward_bias": (_c_int, [_c_int, _c_int, _c_i64, _c_i64, _i64p] + _VIEW + _VIEW + [_ptr]
                                     + _WS + [_ptr]),
     "msd_conv_relu_backward_kb": (_c_int, _HEAD + _VIEW + _VIEW + _VIEW + [_ptr, _ptr] + _WS + [_ptr]),
+    "msd_conv_backward_kb": (_c_int, _HEAD + _VIEW + _VIEW + [_ptr, _ptr] + _WS + [_ptr]),
+    "msd_relu_mask_gradient": (_c_int, [_c_int, _c_int, _c_i64, _c_i64, _i64p] + _VIEW + _VIEW + [_ptr]),
 }
 
 _lib = None

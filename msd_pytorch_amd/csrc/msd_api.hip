@@ -326,6 +326,39 @@ int msd_conv_relu_backward_bias(int dtype, int ndim, int64_t batch, int64_t c_ou
                        workspace, workspace_bytes, stream);
 }
 
+int msd_conv_backward_kb(int dtype, int ndim, int64_t batch, int64_t c_in, int64_t c_out, const int64_t *spatial,
+                         int dilation, const void *grad_output, const int64_t *grad_output_strides, const void *input,
+                         const int64_t *input_strides, void *grad_kernel, void *grad_bias, void *workspace,
+                         int64_t workspace_bytes, void *stream)
+{
+    return backward_kb("conv_backward_kb", false, true, dtype, ndim, batch, c_in, c_out, spatial, dilation, nullptr,
+                       nullptr, grad_output, grad_output_strides, input, input_strides, grad_kernel, grad_bias,
+                       workspace, workspace_bytes, stream);
+}
+
+int msd_relu_mask_gradient(int dtype, int ndim, int64_t batch, int64_t c_out, const int64_t *spatial,
+                           const void *output, const int64_t *output_strides, void *grad_output,
+                           const int64_t *grad_output_strides, void *stream)
+{
+    const char *fn = "relu_mask_gradient";
+    msd::Geom g;
+    MSD_TRY(make_geom(fn, dtype, ndim, batch, 0, c_out, spatial, 1, false, &g));
+    if (dtype == MSD_F32) {
+        msd::View<const float> o;
+        msd::View<float> gy;
+        MSD_TRY(make_view(fn, "output", ndim, output, output_strides, &o));
+        MSD_TRY(make_view(fn, "grad_output", ndim, grad_output, grad_output_strides, &gy));
+        hipError_t e = msd::generic_relu_mask<float>(g, o, gy, (hipStream_t)stream);
+        return e == hipSuccess ? MSD_OK : hip_fail(fn, e);
+    }
+    msd::View<const double> o;
+    msd::View<double> gy;
+    MSD_TRY(make_view(fn, "output", ndim, output, output_strides, &o));
+    MSD_TRY(make_view(fn, "grad_output", ndim, grad_output, grad_output_strides, &gy));
+    hipError_t e = msd::generic_relu_mask<double>(g, o, gy, (hipStream_t)stream);
+    return e == hipSuccess ? MSD_OK : hip_fail(fn, e);
+}
+
 int msd_conv_relu_backward_kb(int dtype, int ndim, int64_t batch, int64_t c_in, int64_t c_out, const int64_t *spatial,
                               int dilation, const void *output, const int64_t *output_strides, const void *grad_output,
                               const int64_t *grad_output_strides, const void *input, const int64_t *input_strides,

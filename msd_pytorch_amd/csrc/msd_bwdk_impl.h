@@ -1,25 +1,33 @@
-// backward_k (+ bias) for fp32 with contiguous rows, on the matrix cores:
+// backward_k (+ bias) for fp32 with unit x-stride, on the matrix cores:
 //     grad_kernel[co][ci][t] += sum_u x[ci][u] * A[co][t](u),   grad_bias[co] += sum_u A[co][centre](u)
-// with A the adjoint-form gather of the masked output gradient (msd_rows.h).
+// with A the adjoint-form gather (msd_adjoint.h) of m = grad_output * [0 < output].
 // Per output channel this is a GEMM  D[tap][channel] = A[tap][voxel] * X[voxel][channel]
 // whose long dimension (voxels) is the contraction, so it maps onto
 // v_mfma_f32_16x16x4_f32 with taps as rows (9 of 16 in 2D, 27 of 2x16 in 3D),
 // 16 input channels as columns and 4 voxels per instruction.
 //
-// A workgroup of four waves walks over tiles of 256*V voxels (rows of the
-// image, row-team mapping).  Per tile it stages the folded source rows in LDS,
-// lets every lane compute the K taps of its own V voxels (as backward_x does),
-// passes them through an LDS tile [tap][voxel] into the MFMA A layout
-// (registers, lane = tap + 16 * voxel) and then streams the input channels in
-// blocks of 16: each wave loads its own
-// 64*V voxels of the 16 channels with coalesced V-wide loads, transposes them
-// through a wave-private LDS tile into the B layout (lane = channel + 16 * voxel)
-// and issues the MFMAs.  The D accumulators stay in registers across all tiles
-// of the workgroup; at the end the four waves are added in LDS and one row of
-// partial sums per workgroup goes to the workspace, which reduce_partials adds
-// up in a fixed order.  A virtual input channel of ones yields the bias sum.
+// Two kernels per call (three with the ReLU mask):
+//   mask_gradient   m = grad_output * [0 < output] into a contiguous scratch plane
+//                   (skipped for the plain operator, which reads grad_output itself);
+//   bwdk_mfma       every WAVE walks its own run of tiles of 64*V consecutive voxels.
+//                   Per tile every lane gathers the K taps of its own V voxels straight
+//                   from m (coalesced, branch-free loads), a wave-private LDS tile
+//                   [tap][voxel] turns them into the MFMA A layout (lane = tap + 16 *
+//                   voxel group, registers); then the wave streams the input channels in
+//                   blocks of 16: coalesced V-wide loads of its 64*V voxels, a
+//                   wave-private LDS tile to turn them into the B layout
+//                   (lane = channel + 16 * voxel group), MFMAs, with the next block's loads
+//                   issued before the MFMAs of the current one.  No workgroup barrier in
+//                   the loop: waves drift freely and hide each other's latencies.  The D
+//                   accumulators stay in registers over all tiles; at the end the four
+//                   waves of a workgroup are added in LDS and one column-major row of
+//                   partial sums per workgroup goes to the workspace;
+//   reduce_columns  adds the partial rows in a fixed order and accumulates into
+//                   grad_kernel / grad_bias.
+// A virtual input channel of ones yields the bias sum.
 // Algorithmic traffic: (C + 2w) * N * 4 bytes.
 #pragma once
+#include "msd_adjoint.h"
 #include "msd_kernels.h"
 #include "msd_rows.h"
 
@@ -34,32 +42,45 @@ constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / kWave;
 constexpr int kChanBlock = 16;
 
+// Wave-private LDS tile: first [tap][voxel] while the A operands are set up,
+// then [channel][voxel] in the channel loop.
 template <int V> struct XTile {
-    static constexpr int kVox = kWave * V;        // voxels per wave
-    static constexpr int kStride = kVox + 4;      // floats per channel row (bank spread for the b128 reads)
-    static constexpr int kFloats = kChanBlock * kStride;
+    static constexpr int kVox = kWave * V;        // voxels per wave tile
+    static constexpr int kStride = kVox + 4;      // floats per row (bank spread for the b128 reads)
+    static constexpr int kRows = 27;              // >= taps (27 in 3D) and >= kChanBlock
+    static constexpr int kFloats = kRows * kStride;
 };
 
-template <int NDIM, bool RELU, int V, int NCB>
-__global__ __launch_bounds__(kThreads, 2) void bwdk_mfma(Geom g, RowTeams rt, int remap, int tiles_per_wg, int ntiles,
-                                                      int groups_per_image, View<const float> out,
-                                                      View<const float> gy, View<const float> x,
-                                                      float *__restrict__ part, int want_bias)
+// m[b][co][voxel] = grad_output * [0 < output], contiguous.
+static __global__ __launch_bounds__(256) void mask_gradient(Geom g, View<const float> out, View<const float> gy,
+                                                            float *__restrict__ m)
+{
+    const int64_t total = (int64_t)g.B * g.Wd * g.nvox;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        const int n = (int)(i % g.nvox);
+        const int64_t bc = i / g.nvox;
+        const int co = (int)(bc % g.Wd), b = (int)(bc / g.Wd);
+        int z, y, x;
+        decode_voxel(g, n, z, y, x);
+        const float o = out.p[(int64_t)b * out.sb + (int64_t)co * out.sc + (int64_t)z * out.sz + (int64_t)y * out.sy + x];
+        const float v = gy.p[(int64_t)b * gy.sb + (int64_t)co * gy.sc + (int64_t)z * gy.sz + (int64_t)y * gy.sy + x];
+        m[i] = 0.f < o ? v : 0.f;
+    }
+}
+
+template <int NDIM, int V, int NCB>
+__global__ __launch_bounds__(kThreads, 2) void bwdk_mfma(Geom g, int remap, int tiles_per_wave, int64_t ntiles,
+                                                         int tiles_per_image, View<const float> m,
+                                                         View<const float> x, float *__restrict__ part,
+                                                         int want_bias)
 {
     extern __shared__ float lds[];
-    constexpr int K = Taps<NDIM>::K, NPQ = RowTaps<NDIM>::NPQ;
+    constexpr int K = Taps<NDIM>::K;
     constexpr int TG = NDIM == 3 ? 2 : 1;         // groups of 16 tap rows
-    constexpr int NS = 4 * V;                     // 16-voxel MFMA groups per wave
+    constexpr int NS = 4 * V;                     // 16-voxel MFMA groups per wave tile
     const int tid = threadIdx.x;
-    const int wave = tid / kWave, wl = tid % kWave;
-    const int team = tid / rt.lpr, lane = tid % rt.lpr;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave), wl = tid % kWave;
     const int mk = wl / 16, mj = wl % 16;         // MFMA k (voxel) and i/j (tap or channel) of this lane
-
-    // LDS: while a tile is set up, S (staged rows) and AL (taps x voxels); in
-    // the channel loop the same memory holds the wave-private input tiles XS.
-    constexpr int TVP = kThreads * V + 4;         // AL row stride (bank spread for the b128 reads)
-    float *S = lds;
-    float *AL = lds + (size_t)NPQ * kThreads * V;
     float *XS = lds + (size_t)wave * XTile<V>::kFloats;
 
     const int co = blockIdx.z % g.Wd;
@@ -67,6 +88,8 @@ __global__ __launch_bounds__(kThreads, 2) void bwdk_mfma(Geom g, RowTeams rt, in
     const int c0 = chunk * NCB * kChanBlock;
     const int ones_ch = want_bias ? g.C : -1;     // virtual channel of ones -> bias sum
     const int c_end = min(g.C + (want_bias ? 1 : 0), c0 + NCB * kChanBlock);
+    const int ncb = (c_end - c0 + kChanBlock - 1) / kChanBlock;
+    const float inv_w = 1.f / (float)g.W, inv_h = 1.f / (float)g.H;
 
     mfma4 D[NCB][TG];
 #pragma unroll
@@ -75,30 +98,38 @@ __global__ __launch_bounds__(kThreads, 2) void bwdk_mfma(Geom g, RowTeams rt, in
         for (int tg = 0; tg < TG; tg++) D[cb][tg] = mfma4{0.f, 0.f, 0.f, 0.f};
 
     const int lb = block_for_xcd(blockIdx.x, gridDim.x, remap);
-    View<const float> out_c = out, gy_c = gy;
-    out_c.p = RELU ? out.p + (int64_t)co * out.sc : nullptr;
-    gy_c.p = gy.p + (int64_t)co * gy.sc;
+    // the four waves of a workgroup take neighbouring tiles, so that together they
+    // read 4 * 64 * V consecutive voxels of every channel at about the same time
+    const int64_t first = (int64_t)lb * kWaves * tiles_per_wave + wave;
 
-    for (int ti = 0; ti < tiles_per_wg; ti++) {
-        const int tile = lb * tiles_per_wg + ti;
-        if (tile >= ntiles) break;                // uniform over the workgroup
+    for (int ti = 0; ti < tiles_per_wave; ti++) {
+        const int64_t t = first + (int64_t)ti * kWaves;
+        if (t >= ntiles) break;                   // uniform over the wave; no workgroup barrier inside the loop
         int64_t xsc = x.sc;
         asm volatile("" : "+s"(xsc));             // keeps the 16 channel offsets from being hoisted out of the loop
-        const int b = tile / groups_per_image;
-        const int row0 = (tile % groups_per_image) * rt.rpw;
-        const int row = row0 + team;
-        const int x0 = lane * V;
-        const bool act = row < rt.nrows && x0 < g.W;
-        const int rr = min(row, rt.nrows - 1);
+        const int b = (int)(t / tiles_per_image);
+        const int n0 = (int)(t % tiles_per_image) * XTile<V>::kVox;
+        // position of the first voxel of the tile; everything else is a small offset from it
+        const int row0 = n0 / g.W, xb = n0 % g.W;
+        const int yb = row0 % g.H, zb = row0 / g.H;
+        auto locate = [&](int off, int &z, int &y, int &xx) {
+            const int xs = xb + off;                               // < W + 256: the float quotient is exact
+            const int q = (int)(((float)xs + 0.5f) * inv_w);
+            xx = xs - q * g.W;
+            const int ys = yb + q;
+            const int qz = (int)(((float)ys + 0.5f) * inv_h);
+            y = ys - qz * g.H;
+            z = zb + qz;
+        };
 
-        const float *xp0 = x.p + (int64_t)b * x.sb + (int64_t)(rr / g.H) * x.sz + (int64_t)(rr % g.H) * x.sy +
-                           min(x0, g.W - V);
-        const int ncb = (c_end - c0 + kChanBlock - 1) / kChanBlock;
-        // Input values of 16 channels for this lane's voxels.  Branch-free: every
-        // lane loads from a clamped, valid address, so all 16 loads are in flight
-        // together; values that must not count are replaced in fix_block().
+        // ---- input values of 16 channels for this lane's V voxels (B operand, before the transpose)
+        const bool act = n0 + wl * V < g.nvox;
+        int lz, ly, lx;
+        locate(min(wl * V, g.nvox - V - n0), lz, ly, lx);
+        const float *xp0 = x.p + (int64_t)b * x.sb + (int64_t)lz * x.sz + (int64_t)ly * x.sy + lx;
         float xv[kChanBlock][V];
         auto load_block = [&](int cb) {
+            // branch-free: clamped channel index, all 16 loads in flight together
 #pragma unroll
             for (int c = 0; c < kChanBlock; c++)
                 load_vec<V>(xp0 + (int64_t)min(c0 + cb * kChanBlock + c, g.C - 1) * xsc, xv[c]);
@@ -113,39 +144,75 @@ __global__ __launch_bounds__(kThreads, 2) void bwdk_mfma(Geom g, RowTeams rt, in
                 for (int i = 0; i < V; i++) xv[c][i] = keep ? xv[c][i] : fill;
             }
         };
-        load_block(0);   // issued ahead of the set-up so its latency overlaps with it
+        load_block(0);   // issued ahead of the gather so the two latencies overlap
 
+        // ---- A operands.  Step 1, voxel layout: every lane gathers the K taps of its own V
+        // voxels from m.  Consecutive lanes read consecutive addresses (coalesced); all loads
+        // go to clamped, always valid addresses and are masked afterwards, so there is no
+        // branch around them and they are all in flight together.
+        const float *mc = m.p + (int64_t)b * m.sb + (int64_t)co * m.sc;
         {
-            float own[1][NPQ][V];
-            float *srows = S + (size_t)team * NPQ * V * rt.lpr;
-            stage_source_rows<NDIM, RELU, 1, V>(g, rt, out_c, gy_c, b, rr / g.H, rr % g.H, lane, act, srows, own);
-            // the K taps of this lane's V voxels -> AL[tap][tid * V + i]
-            float t[NPQ][3][V];
+            const AxisSources sz = NDIM == 3 ? adjoint_sources(lz, g.D, g.dil) : single_source();
+            const AxisSources sy = adjoint_sources(ly, g.H, g.dil);
+            // x sources of voxel lx + i: tap 0 reads x + dil (and the fold partner dil - x - 1),
+            // tap 2 reads x - dil (and 2W - x - 1 - dil)
+            int c0a[V], c0b[V], c2a[V], c2b[V];
+            bool k0a[V], k0b[V], k2a[V], k2b[V];
 #pragma unroll
             for (int i = 0; i < V; i++) {
-                const SideTaps<V> side(x0 + i, g.W, g.dil, rt.lpr);
+                const int xx = lx + i;
+                c0a[i] = min(xx + g.dil, g.W - 1);                        k0a[i] = xx + g.dil < g.W;
+                c0b[i] = max(g.dil - xx - 1, 0);                          k0b[i] = xx < g.dil;
+                c2a[i] = max(xx - g.dil, 0);                              k2a[i] = xx >= g.dil;
+                c2b[i] = min(max(2 * g.W - xx - 1 - g.dil, 0), g.W - 1);  k2b[i] = xx + g.dil >= g.W;
+            }
+            float tv[K][V];
+            auto add_rows = [&](int a_, int b_, bool first) {
 #pragma unroll
-                for (int pq = 0; pq < NPQ; pq++) {
-                    side.read(srows + (size_t)pq * V * rt.lpr, t[pq][0][i], t[pq][2][i]);
-                    t[pq][1][i] = own[0][pq][i];
+                for (int p = 0; p < Taps<NDIM>::NZ; p++)
+#pragma unroll
+                    for (int q = 0; q < 3; q++) {
+                        const int pz = NDIM == 3 ? p : 0;
+                        const int cz = min(max(sz.c[pz][a_], 0), g.D - 1), cy = min(max(sy.c[q][b_], 0), g.H - 1);
+                        const bool use = act && sz.ok[pz][a_] && sy.ok[q][b_];
+                        const float *row = mc + (int64_t)cz * m.sz + (int64_t)cy * m.sy;
+                        float mid[V];
+                        load_vec<V>(row + lx, mid);
+#pragma unroll
+                        for (int i = 0; i < V; i++) {
+                            const float v0a = row[c0a[i]], v0b = row[c0b[i]], v2a = row[c2a[i]], v2b = row[c2b[i]];
+                            const float t0 = (use && k0a[i] ? v0a : 0.f) + (use && k0b[i] ? v0b : 0.f);
+                            const float t1 = use ? mid[i] : 0.f;
+                            const float t2 = (use && k2a[i] ? v2a : 0.f) + (use && k2b[i] ? v2b : 0.f);
+                            const int t = (p * 3 + q) * 3;
+                            tv[t + 0][i] = first ? t0 : tv[t + 0][i] + t0;
+                            tv[t + 1][i] = first ? t1 : tv[t + 1][i] + t1;
+                            tv[t + 2][i] = first ? t2 : tv[t + 2][i] + t2;
+                        }
+                    }
+            };
+            add_rows(0, 0, true);
+            const bool folds = ly < g.dil || ly + g.dil >= g.H || (NDIM == 3 && (lz < g.dil || lz + g.dil >= g.D));
+            if (folds) {   // rows within dil of a y or z border: the fold maps a second row onto some taps
+                add_rows(0, 1, false);
+                if (NDIM == 3) {
+                    add_rows(1, 0, false);
+                    add_rows(1, 1, false);
                 }
             }
+            // Step 2: through a wave-private LDS tile [tap][voxel] into the MFMA layout.
 #pragma unroll
-            for (int pq = 0; pq < NPQ; pq++)
-#pragma unroll
-                for (int r = 0; r < 3; r++) {
-#pragma unroll
-                    for (int i = 0; i < V; i++) t[pq][r][i] = act ? t[pq][r][i] : 0.f;
-                    store_vec<V>(AL + (size_t)(pq * 3 + r) * TVP + tid * V, t[pq][r]);
-                }
+            for (int t = 0; t < K; t++) store_vec<V>(XS + t * XTile<V>::kStride + wl * V, tv[t]);
         }
-        __syncthreads();
-        // A operands: a[tg][s][e] = A[tap = tg*16 + mj](voxel wave*64V + 16 s + 4 mk + e)
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        // a[tg][s][e] = A[tap = tg*16 + mj](voxel n0 + 16 s + 4 mk + e)
         float a[TG][NS][4];
 #pragma unroll
         for (int tg = 0; tg < TG; tg++) {
             const int tap = tg * 16 + mj;
-            const float *arow = AL + (size_t)min(tap, K - 1) * TVP + wave * XTile<V>::kVox + 4 * mk;
+            const float *arow = XS + min(tap, K - 1) * XTile<V>::kStride + 4 * mk;
 #pragma unroll
             for (int s = 0; s < NS; s++) {
                 const f32x4 av = *reinterpret_cast<const f32x4 *>(arow + 16 * s);
@@ -153,13 +220,14 @@ __global__ __launch_bounds__(kThreads, 2) void bwdk_mfma(Geom g, RowTeams rt, in
                 for (int e = 0; e < 4; e++) a[tg][s][e] = tap < K ? av[e] : 0.f;
             }
         }
-        __syncthreads();   // S and AL are dead from here on: the channel loop reuses their memory
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
-        // runtime loop: unrolled, the per-channel addresses and predicates of all
-        // NCB blocks would be computed up front and spill
+        // ---- channel loop.  Runtime loop: unrolled, the per-channel addresses and predicates of
+        // all NCB blocks would be computed up front and spill.
 #pragma unroll 1
         for (int cb = 0; cb < ncb; cb++) {
-            // this wave's 64*V voxels of 16 channels -> wave-private LDS tile [channel][voxel]
             fix_block(cb);
 #pragma unroll
             for (int c = 0; c < kChanBlock; c++) store_vec<V>(XS + c * XTile<V>::kStride + wl * V, xv[c]);
@@ -193,7 +261,6 @@ __global__ __launch_bounds__(kThreads, 2) void bwdk_mfma(Geom g, RowTeams rt, in
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         }
-        __syncthreads();   // all waves are done with their tiles before the next set-up reuses the memory
     }
 
     // D[cb][tg][v] = sum for tap tg*16 + 4*mk + v, channel c0 + cb*16 + mj.  Add the four waves in LDS.
@@ -249,76 +316,71 @@ static __global__ __launch_bounds__(256) void reduce_columns(const float *__rest
     }
 }
 
-constexpr size_t kMaxLds = 160 * 1024;   // LDS per CU on gfx950; above 64 KB a kernel must opt in
-
 template <int NDIM, int V, int NCB>
 size_t lds_bytes()
 {
     constexpr int TG = NDIM == 3 ? 2 : 1;
-    const size_t setup = ((size_t)RowTaps<NDIM>::NPQ * kThreads * V + (size_t)Taps<NDIM>::K * (kThreads * V + 4)) * 4;
     const size_t main_loop = (size_t)kWaves * XTile<V>::kFloats * 4;
     const size_t epilogue = (size_t)kWaves * NCB * TG * 4 * kWave * 4;
-    return std::max(setup, std::max(main_loop, epilogue));
+    return std::max(main_loop, epilogue);
 }
 
-template <int NDIM, bool RELU, int V, int NCB>
-hipError_t launch(const Geom &g, const View<const float> &out, const View<const float> &gy,
+template <int NDIM, int V, int NCB>
+hipError_t launch(const Geom &g, bool relu, const View<const float> &out, const View<const float> &gy,
                   const View<const float> &x, float *gk, float *gb, float *ws, hipStream_t s)
 {
     constexpr int K = Taps<NDIM>::K;
-    RowTeams rt;
-    make_row_teams(g, V, &rt);
-    const int groups = (rt.nrows + rt.rpw - 1) / rt.rpw;
-    const int ntiles = groups * g.B;
+    View<const float> m = gy;
+    float *part = ws;
+    if (relu) {
+        float *mbuf = ws;
+        part = ws + backward_k_mask_floats(g);
+        const int64_t total = (int64_t)g.B * g.Wd * g.nvox;
+        const int blocks = (int)std::min<int64_t>((total + 255) / 256, 4096);
+        hipLaunchKernelGGL(mask_gradient, dim3(blocks), dim3(256), 0, s, g, out, gy, mbuf);
+        m = View<const float>{mbuf, (int64_t)g.Wd * g.nvox, (int64_t)g.nvox, (int64_t)g.H * g.W, (int64_t)g.W, 1};
+    }
+    const int tiles_per_image = (g.nvox + XTile<V>::kVox - 1) / XTile<V>::kVox;
+    const int64_t ntiles = (int64_t)tiles_per_image * g.B;
     const int remap = knob(kKnobXcdRemap, 1);
-    int wgs = min(ntiles, knob(kKnobBwdkBlocks, kMaxPartialRows));
-    wgs = min(wgs, kMaxPartialRows);
-    const int tiles_per_wg = (ntiles + wgs - 1) / wgs;
-    wgs = (ntiles + tiles_per_wg - 1) / tiles_per_wg;
-    const int rows = remap ? xcd_grid(wgs) : wgs;   // padding workgroups write zero rows
+    int64_t wgs = std::min<int64_t>((ntiles + kWaves - 1) / kWaves, knob(kKnobBwdkBlocks, kMaxPartialRows));
+    wgs = std::min<int64_t>(wgs, kMaxPartialRows);
+    const int tiles_per_wave = (int)((ntiles + wgs * kWaves - 1) / (wgs * kWaves));
+    wgs = (ntiles + (int64_t)tiles_per_wave * kWaves - 1) / ((int64_t)tiles_per_wave * kWaves);
+    const int rows = remap ? xcd_grid((int)wgs) : (int)wgs;   // padding workgroups write zero rows
     if (rows > kMaxPartialRows) return hipErrorInvalidConfiguration;
     const int want_bias = gb != nullptr;
     const int chunks = (g.C + want_bias + NCB * kChanBlock - 1) / (NCB * kChanBlock);
     const size_t lds = lds_bytes<NDIM, V, NCB>();
-    if (lds > 64 * 1024) {
-        static const hipError_t attr = hipFuncSetAttribute(
-            reinterpret_cast<const void *>(&bwdk_mfma<NDIM, RELU, V, NCB>),
-            hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds);
-        if (attr != hipSuccess) return attr;
-    }
-    hipLaunchKernelGGL((bwdk_mfma<NDIM, RELU, V, NCB>), dim3(rows, 1, chunks * g.Wd), dim3(kThreads), lds, s, g, rt,
-                       remap, tiles_per_wg, ntiles, groups, out, gy, x, ws, want_bias);
+    hipLaunchKernelGGL((bwdk_mfma<NDIM, V, NCB>), dim3(rows, 1, chunks * g.Wd), dim3(kThreads), lds, s, g, remap,
+                       tiles_per_wave, ntiles, tiles_per_image, m, x, part, want_bias);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     const int64_t nk = (int64_t)g.Wd * g.C * K;
     const int64_t ncols = nk + (want_bias ? g.Wd : 0);
-    hipLaunchKernelGGL(reduce_columns, dim3((ncols + 3) / 4), dim3(256), 0, s, ws, rows, nk, ncols, gk, gb);
+    hipLaunchKernelGGL(reduce_columns, dim3((ncols + 3) / 4), dim3(256), 0, s, part, rows, nk, ncols, gk, gb);
     return hipGetLastError();
 }
 
-template <int NDIM, bool RELU, int V>
-hipError_t pick_ncb(const Geom &g, const View<const float> &out, const View<const float> &gy,
+template <int NDIM, int V>
+hipError_t pick_ncb(const Geom &g, bool relu, const View<const float> &out, const View<const float> &gy,
                     const View<const float> &x, float *gk, float *gb, float *ws, hipStream_t s)
 {
     const int need = (g.C + (gb != nullptr) + kChanBlock - 1) / kChanBlock;
-    if (need <= 1) return launch<NDIM, RELU, V, 1>(g, out, gy, x, gk, gb, ws, s);
-    if (need <= 2) return launch<NDIM, RELU, V, 2>(g, out, gy, x, gk, gb, ws, s);
-    if (need <= 4) return launch<NDIM, RELU, V, 4>(g, out, gy, x, gk, gb, ws, s);
-    return launch<NDIM, RELU, V, 8>(g, out, gy, x, gk, gb, ws, s);
+    if (need <= 1) return launch<NDIM, V, 1>(g, relu, out, gy, x, gk, gb, ws, s);
+    if (need <= 2) return launch<NDIM, V, 2>(g, relu, out, gy, x, gk, gb, ws, s);
+    if (need <= 4) return launch<NDIM, V, 4>(g, relu, out, gy, x, gk, gb, ws, s);
+    return launch<NDIM, V, 8>(g, relu, out, gy, x, gk, gb, ws, s);
 }
 
-// Voxels per lane: V-wide accesses aligned in every view and a tile of
-// 256 * V voxels made of whole rows (row-team mapping with 256 lanes).
-template <int NDIM>
-int choose_vec(const Geom &g, bool relu, int vmax, const View<const float> &out, const View<const float> &gy,
-               const View<const float> &x)
+// Voxels per lane: V-wide accesses to the input must be aligned, and groups of
+// four consecutive voxels must not straddle rows (W % 4 == 0).
+inline int choose_vec(const Geom &g, int vmax, const View<const float> &x)
 {
-    for (int v = 4; v >= 1; v /= 2) {
+    if (g.W % 4 != 0 || g.nvox < 4) return 0;
+    for (int v = 4; v >= 2; v /= 2) {
         if (v > vmax) continue;
-        if (!rows_aligned(x, g.W, v) || !rows_aligned(gy, g.W, v) || (relu && !rows_aligned(out, g.W, v))) continue;
-        RowTeams rt;
-        if (!make_row_teams(g, v, &rt) || rt.lpr * rt.rpw != kThreads) continue;
-        return v;
+        if (rows_aligned(x, g.W, v)) return v;
     }
     return 0;
 }
@@ -328,28 +390,19 @@ bool supported_nd(const Geom &g, bool relu, const View<const float> &out, const 
                   const View<const float> &x)
 {
     if (x.sx != 1 || gy.sx != 1 || (relu && out.sx != 1)) return false;
-    return choose_vec<NDIM>(g, relu, 4, out, gy, x) != 0;
-}
-
-template <int NDIM, bool RELU>
-hipError_t pick_vec(const Geom &g, const View<const float> &out, const View<const float> &gy,
-                    const View<const float> &x, float *gk, float *gb, float *ws, hipStream_t s)
-{
-    const int vmax = knob(NDIM == 3 ? kKnobBwdkVec3d : kKnobBwdkVec2d, NDIM == 3 ? 2 : 4);
-    int v = choose_vec<NDIM>(g, RELU, vmax, out, gy, x);
-    if (v == 0) v = choose_vec<NDIM>(g, RELU, 4, out, gy, x);
-    if (v == 4) return pick_ncb<NDIM, RELU, 4>(g, out, gy, x, gk, gb, ws, s);
-    if (v == 2) return pick_ncb<NDIM, RELU, 2>(g, out, gy, x, gk, gb, ws, s);
-    if (v == 1) return pick_ncb<NDIM, RELU, 1>(g, out, gy, x, gk, gb, ws, s);
-    return hipErrorInvalidConfiguration;
+    return choose_vec(g, 4, x) != 0;
 }
 
 template <int NDIM>
 hipError_t run_nd(const Geom &g, bool relu, const View<const float> &out, const View<const float> &gy,
                   const View<const float> &x, float *gk, float *gb, float *ws, hipStream_t s)
 {
-    return relu ? pick_vec<NDIM, true>(g, out, gy, x, gk, gb, ws, s)
-                : pick_vec<NDIM, false>(g, out, gy, x, gk, gb, ws, s);
+    const int vmax = knob(NDIM == 3 ? kKnobBwdkVec3d : kKnobBwdkVec2d, NDIM == 3 ? 2 : 4);
+    int v = choose_vec(g, vmax, x);
+    if (v == 0) v = choose_vec(g, 4, x);
+    if (v == 4) return pick_ncb<NDIM, 4>(g, relu, out, gy, x, gk, gb, ws, s);
+    if (v == 2) return pick_ncb<NDIM, 2>(g, relu, out, gy, x, gk, gb, ws, s);
+    return hipErrorInvalidConfiguration;
 }
 
 }  // namespace bwdk

@@ -199,6 +199,25 @@ __global__ __launch_bounds__(kBlock) void reduce_partials(const T *__restrict__ 
     dst[i] += s;
 }
 
+// gy = gy * [0 < out], in place, over batch * Wd * nvox elements.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void relu_mask_inplace(Geom g, View<const T> out, View<T> gy)
+{
+    const int64_t total = (int64_t)g.B * g.Wd * g.nvox;
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += (int64_t)gridDim.x * kBlock) {
+        const int n = (int)(i % g.nvox);
+        const int64_t bc = i / g.nvox;
+        const int co = (int)(bc % g.Wd), b = (int)(bc / g.Wd);
+        int z, y, x;
+        decode_voxel(g, n, z, y, x);
+        const T o = out.p[(int64_t)b * out.sb + (int64_t)co * out.sc + (int64_t)z * out.sz + (int64_t)y * out.sy +
+                          (int64_t)x * out.sx];
+        T *p = gy.p + (int64_t)b * gy.sb + (int64_t)co * gy.sc + (int64_t)z * gy.sz + (int64_t)y * gy.sy +
+               (int64_t)x * gy.sx;
+        if (!(T(0) < o)) *p = T(0);
+    }
+}
+
 inline int partial_rows(const Geom &g)
 {
     const int64_t total = (int64_t)g.B * g.nvox;
@@ -266,7 +285,7 @@ int64_t generic_workspace_elems(const Geom &g)
 {
     const int K = g.ndim == 3 ? 27 : 9;
     // sized for the largest row count any backward_k path uses
-    return (int64_t)kMaxPartialRows * ((int64_t)g.Wd * g.C * K + g.Wd);
+    return backward_k_mask_floats(g) + (int64_t)kMaxPartialRows * ((int64_t)g.Wd * g.C * K + g.Wd);
 }
 
 template <typename T>
@@ -298,11 +317,21 @@ hipError_t generic_backward_kb(const Geom &g, bool relu, View<const T> out, View
                 : launch_bwdk<T, 3, false>(g, out, gy, x, gk, gb, ws, s);
 }
 
+template <typename T>
+hipError_t generic_relu_mask(const Geom &g, View<const T> out, View<T> gy, hipStream_t s)
+{
+    const int64_t total = (int64_t)g.B * g.Wd * g.nvox;
+    const int blocks = (int)((total + kBlock - 1) / kBlock < 8192 ? (total + kBlock - 1) / kBlock : 8192);
+    hipLaunchKernelGGL((relu_mask_inplace<T>), dim3(blocks), dim3(kBlock), 0, s, g, out, gy);
+    return hipGetLastError();
+}
+
 #define MSD_INSTANTIATE(T)                                                                                         \
     template hipError_t generic_forward<T>(const Geom &, bool, View<const T>, const T *, const T *, View<T>,       \
                                            hipStream_t);                                                           \
     template hipError_t generic_backward_x<T>(const Geom &, bool, View<const T>, View<const T>, const T *, View<T>, \
                                               hipStream_t);                                                        \
+    template hipError_t generic_relu_mask<T>(const Geom &, View<const T>, View<T>, hipStream_t);                     \
     template hipError_t generic_backward_kb<T>(const Geom &, bool, View<const T>, View<const T>, View<const T>,    \
                                                T *, T *, T *, hipStream_t);
 MSD_INSTANTIATE(float)

@@ -9,7 +9,12 @@ namespace msd {
 // reduction (one row per workgroup of the first pass).
 constexpr int kMaxPartialRows = 512;
 
-// Scratch elements needed by generic_backward_kb for this geometry.
+// Elements at the start of the workspace that hold the masked output gradient
+// of the matrix-core backward_k (a multiple of 64 so the partial sums behind it
+// stay aligned).
+inline int64_t backward_k_mask_floats(const Geom &g) { return ((int64_t)g.B * g.Wd * g.nvox + 63) / 64 * 64; }
+
+// Scratch elements any backward_k / backward_bias path needs for this geometry.
 int64_t generic_workspace_elems(const Geom &g);
 
 template <typename T>
@@ -19,6 +24,10 @@ hipError_t generic_forward(const Geom &g, bool relu, View<const T> x, const T *k
 template <typename T>
 hipError_t generic_backward_x(const Geom &g, bool relu, View<const T> out, View<const T> gy, const T *k, View<T> gx,
                               hipStream_t s);
+
+// gy = gy * [0 < out] in place.
+template <typename T>
+hipError_t generic_relu_mask(const Geom &g, View<const T> out, View<T> gy, hipStream_t s);
 
 // gk and/or gb may be null (that gradient is then skipped).
 template <typename T>

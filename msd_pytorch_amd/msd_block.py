@@ -61,14 +61,19 @@ class MSDBlockFunction(torch.autograd.Function):
             out_i, gout_i = stack[:, first:last], grads[:, first:last]
             dilation = ctx.dilations[idx]
 
+            # `grads` is private to this call and the layer's slice is not read again
+            # afterwards, so the ReLU mask is applied to it once, in place, and the
+            # plain operators do the rest (the reference masks on the fly in each of
+            # conv_relu_backward_x / _k / _bias, msd_block.py:107-126).
+            cc.relu_mask_gradient(out_i, gout_i)
             if idx > 0 or need_input:
-                cc.conv_relu_backward_x(out_i, gout_i, weight, grads[:, :first], dilation)
+                cc.conv_backward_x(gout_i, weight, grads[:, :first], dilation)
             if need_weights[idx]:
                 grad_weights[idx] = torch.zeros_like(weight)
-                cc.conv_relu_backward_kb(out_i, gout_i, stack[:, :first], grad_weights[idx],
-                                         grad_bias[b0:b1] if need_bias else None, dilation)
+                cc.conv_backward_kb(gout_i, stack[:, :first], grad_weights[idx],
+                                    grad_bias[b0:b1] if need_bias else None, dilation)
             elif need_bias:
-                cc.conv_relu_backward_bias(out_i, gout_i, grad_bias[b0:b1])
+                cc.conv_backward_bias(gout_i, grad_bias[b0:b1])
             last, b1 = first, b0
 
         grad_input = grads[:, :weights[0].shape[1]] if need_input else None

@@ -225,7 +225,7 @@ def _backward_k(fn, native, output, grad_output, input, grad_kernel, grad_bias, 
     head = _head(input, c_in, c_out, dilation)
     views = (*_view(output),) if relu else ()
     grads = (ctypes.c_void_p(grad_kernel.data_ptr()),)
-    if native == "msd_conv_relu_backward_kb":
+    if native in ("msd_conv_relu_backward_kb", "msd_conv_backward_kb"):
         grads += (ctypes.c_void_p(grad_bias.data_ptr() if grad_bias is not None else 0),)
     _call(native, input.device, *head, *views, *_view(grad_output), *_view(input), *grads, ws_ptr, ws_bytes,
           _stream(input))
@@ -248,6 +248,27 @@ def conv_relu_backward_kb(output, grad_output, input, grad_kernel, grad_bias, di
     calls msd_block.py:113-126 makes per layer).  Not part of the reference's module."""
     _backward_k("conv_relu_backward_kb", "msd_conv_relu_backward_kb", output, grad_output, input, grad_kernel,
                 grad_bias, dilation, block_size)
+
+
+def conv_backward_kb(grad_output, input, grad_kernel, grad_bias, dilation, block_size=None):
+    """conv_backward_k and conv_backward_bias in one pass.  Not part of the reference's module."""
+    _backward_k("conv_backward_kb", "msd_conv_backward_kb", None, grad_output, input, grad_kernel, grad_bias,
+                dilation, block_size)
+
+
+def relu_mask_gradient(output, grad_output):
+    """grad_output *= (output > 0), in place: the mask the three conv_relu_backward_*
+    operators of a layer apply on the fly, applied once (for callers that own
+    grad_output, like the dense block's private gradient stack).  Not part of the
+    reference's module."""
+    fn = "relu_mask_gradient"
+    _check_same_gpu(fn, [("output", output), ("grad_output", grad_output)])
+    _check_same_type(fn, [("output", output), ("grad_output", grad_output)])
+    if tuple(output.shape) != tuple(grad_output.shape) or output.dim() not in (4, 5):
+        _fail(fn, "output and grad_output must be 4- or 5-dimensional tensors of the same shape")
+    _call("msd_relu_mask_gradient", output.device, _DTYPES[output.dtype], output.dim() - 2, output.shape[0],
+          output.shape[1], _native.i64_array(tuple(output.shape[2:])), *_view(output), *_view(grad_output),
+          _stream(output))
 
 
 def _backward_bias(fn, native, output, grad_output, grad_bias, block_size):

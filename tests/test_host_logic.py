@@ -33,6 +33,16 @@ def oracle_ops(monkeypatch):
             oracle.conv_relu_backward_bias(output, grad_output, grad_bias)
     monkeypatch.setattr(cc, "conv_relu_backward_kb", kb)
 
+    def plain_kb(grad_output, input, grad_kernel, grad_bias, dilation, block_size=None):
+        oracle.conv_backward_k(grad_output, input, grad_kernel, dilation)
+        if grad_bias is not None:
+            oracle.conv_backward_bias(grad_output, grad_bias)
+    monkeypatch.setattr(cc, "conv_backward_kb", plain_kb)
+
+    def mask(output, grad_output):
+        grad_output.mul_((output > 0).to(grad_output.dtype))
+    monkeypatch.setattr(cc, "relu_mask_gradient", mask)
+
 
 def test_top_level_alias_of_the_native_module():
     import msd_custom_convolutions   # the name the reference's Python layers import (conv2d.py:5)

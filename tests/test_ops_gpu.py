@@ -139,3 +139,26 @@ def test_dtype_and_device_errors(cc):
         cc.conv_relu_forward(x, torch.zeros(1, 1, 3, 6, device="cuda")[..., ::2], b, y, 1)   # non-contiguous kernel
     with pytest.raises(RuntimeError):
         cc.conv_relu_forward(x, torch.zeros(1, 2, 3, 3, device="cuda"), b, y, 1)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("shape", [ALL_SHAPES[5], ALL_SHAPES[10], SHAPES_FAST[3], SHAPES_FAST[8]])
+def test_mask_once_then_plain_operators(cc, shape, dtype):
+    # masking the gradient in place and calling the plain operators (what the dense
+    # block does) equals the three conv_relu_backward_* operators
+    p = make_problem(shape, dtype, device="cuda")
+    cc.conv_relu_forward(p["x"], p["k"], p["bias"], p["y"], p["d"])
+    gx0 = p["gx"].clone()
+    gk0, gb0 = torch.zeros_like(p["k"]), torch.zeros_like(p["bias"])
+    cc.conv_relu_backward_x(p["y"], p["gy"], p["k"], gx0, p["d"])
+    cc.conv_relu_backward_kb(p["y"], p["gy"], p["x"], gk0, gb0, p["d"])
+
+    gy = p["gy"].clone()
+    cc.relu_mask_gradient(p["y"], gy)
+    assert torch.equal(gy, p["gy"] * (p["y"] > 0))
+    gx1 = p["gx"].clone()
+    gk1, gb1 = torch.zeros_like(p["k"]), torch.zeros_like(p["bias"])
+    cc.conv_backward_x(gy, p["k"], gx1, p["d"])
+    cc.conv_backward_kb(gy, p["x"], gk1, gb1, p["d"])
+    tol = 1e-5 if dtype == torch.float32 else 1e-12
+    assert rel_err(gx1, gx0) <= tol and rel_err(gk1, gk0) <= tol and rel_err(gb1, gb0) <= tol
