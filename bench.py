@@ -23,6 +23,12 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 
+# HBM-side bytes per step of each kernel class from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE (summaries and commands under profiles/), each scaled by what the same
+# counter reads for a 1 GiB device copy in the same run (FETCH_SIZE x 2.000,
+# WRITE_SIZE x 1.000).  Filled in from the committed profiles; None = not measured.
+TRAFFIC = {}
+
 WORKLOADS = {
     # name: (kind, ndim, c_in, c_out/labels, depth, width, batch, spatial, adam)
     "A": ("regression", 2, 1, 1, 10, 1, 1, (256, 256), False),
@@ -91,43 +97,22 @@ def algorithmic_bytes(name):
     return out, n
 
 
-class KernelTimer:
-    """Wraps the operator entry points with HIP events recorded on the current
-    (launch) stream; durations are read after a final synchronise."""
-
-    # the dense block applies the ReLU mask to its gradient stack once per layer
-    # (relu_mask_gradient, timed with backward_x, whose on-the-fly mask it replaces)
-    # and then calls the plain backward operators
-    NAMES = {"conv_relu_forward": "forward", "relu_mask_gradient": "backward_x", "conv_backward_x": "backward_x",
-             "conv_backward_kb": "backward_kb"}
-
-    def __init__(self, torch, cc):
-        self.torch, self.cc = torch, cc
-        self.events = {v: [] for v in self.NAMES.values()}
-        self.saved = {}
-
-    def __enter__(self):
-        for fn, cls in self.NAMES.items():
-            orig = getattr(self.cc, fn)
-            self.saved[fn] = orig
-
-            def timed(*a, _orig=orig, _cls=cls, **kw):
-                e0 = self.torch.cuda.Event(enable_timing=True)
-                e1 = self.torch.cuda.Event(enable_timing=True)
-                e0.record()
-                _orig(*a, **kw)
-                e1.record()
-                self.events[_cls].append((e0, e1))
-            setattr(self.cc, fn, timed)
-        return self
-
-    def __exit__(self, *exc):
-        for fn, orig in self.saved.items():
-            setattr(self.cc, fn, orig)
-
-    def totals_ms(self):
-        self.torch.cuda.synchronize()
-        return {cls: (sum(a.elapsed_time(b) for a, b in evs), len(evs)) for cls, evs in self.events.items()}
+def kernel_times(lib, torch, run_steps):
+    """Per-class kernel time of `run_steps()`: the library brackets every operator
+    launch with HIP events recorded on the launch stream (msd_profile_enable) and
+    msd_profile_read sums the elapsed times after a synchronise."""
+    import ctypes
+    lib.msd_profile_enable(1)
+    run_steps()
+    torch.cuda.synchronize()
+    ms = (ctypes.c_double * 3)()
+    calls = (ctypes.c_int64 * 3)()
+    rc = lib.msd_profile_read(ms, calls)
+    lib.msd_profile_enable(0)
+    if rc != 0:
+        raise RuntimeError(lib.msd_last_error().decode())
+    names = ("forward", "backward_x", "backward_kb")
+    return {n: (ms[i], calls[i]) for i, n in enumerate(names)}
 
 
 def cpu_baseline(name, budget_s=20.0):
@@ -184,8 +169,7 @@ def main():
 
     import torch
     from msd_pytorch_amd import _native
-    from msd_pytorch_amd import msd_custom_convolutions as cc
-    _native.load()
+    lib = _native.load()
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
 
@@ -234,10 +218,7 @@ def main():
     }
 
     if not args.no_kernel_timing:
-        with KernelTimer(torch, cc) as kt:
-            for _ in range(args.steps):
-                step()
-            totals = kt.totals_ms()
+        totals = kernel_times(lib, torch, lambda: [step() for _ in range(args.steps)])
         kernels = {}
         for cls, (ms, launches) in totals.items():
             if launches == 0:
@@ -252,8 +233,9 @@ def main():
         dominant = max(kernels, key=lambda c: kernels[c]["ms_per_step"])
         result["roofline"] = {"bound": "hbm", "kernel": dominant, "achieved": kernels[dominant]["GBps"],
                               "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": kernels[dominant]["frac_hbm"],
-                              "traffic": None,
-                              "timed": "HIP events on the launch stream, instrumented repeat of the K steps"}
+                              "traffic": TRAFFIC.get(name, {}).get(dominant),
+                              "timed": "HIP events on the launch stream around every operator launch "
+                                       "(msd_profile_enable), in a repeat of the K timed steps"}
         result["kernels"] = kernels
         hot = sum(k["ms_per_step"] for k in kernels.values())
         result["hot_path_ms_per_step"] = round(hot, 4)

@@ -184,6 +184,49 @@ int msd_relu_mask_gradient(int dtype, int ndim, int64_t batch, int64_t c_out, co
                            const void *output, const int64_t *output_strides,
                            void *grad_output, const int64_t *grad_output_strides, void *stream);
 
+/*
+ * Dense block (MSDBlockFunction, msd_block.py:8-134) as one call per direction.
+ * `stack` is the (batch, c_in + sum(widths), spatial) channel stack; layer i reads
+ * channels [0, C_i) and writes [C_i, C_i + widths[i]), C_i = c_in + widths[0..i).
+ * `weights[i]` is the contiguous (widths[i], C_i, 3, 3[, 3]) kernel of layer i
+ * (host array of device pointers), `bias` the flat bias of sum(widths) entries.
+ *
+ * msd_block_forward: channels [0, c_in) of `stack` hold the input on entry; the
+ * remaining channels are computed (the loop of msd_block.py:40-58).
+ *
+ * msd_block_backward: `grads` holds dL/dstack on entry and is MODIFIED IN PLACE (it
+ * is the private working copy of msd_block.py:83); on return channels [0, c_in) hold
+ * dL/dinput (if need_input_grad).  grad_weights[i] (zero-filled by the caller, NULL to
+ * skip a layer) and grad_bias (zero-filled, NULL to skip) are accumulated into.
+ * Replaces the loop of msd_block.py:89-130.  Workspace: msd_block_workspace_bytes.
+ */
+int64_t msd_block_workspace_bytes(int dtype, int ndim, int64_t batch, int64_t c_in, int depth,
+                                  const int64_t *widths, const int64_t *spatial);
+
+int msd_block_forward(int dtype, int ndim, int64_t batch, int64_t c_in, int depth, const int64_t *widths,
+                      const int64_t *spatial, const int64_t *dilations,
+                      void *stack, const int64_t *stack_strides,
+                      const void *const *weights, const void *bias, void *stream);
+
+int msd_block_backward(int dtype, int ndim, int64_t batch, int64_t c_in, int depth, const int64_t *widths,
+                       const int64_t *spatial, const int64_t *dilations,
+                       const void *stack, const int64_t *stack_strides,
+                       void *grads, const int64_t *grads_strides,
+                       const void *const *weights, void *const *grad_weights, void *grad_bias,
+                       int need_input_grad,
+                       void *workspace, int64_t workspace_bytes, void *stream);
+
+/*
+ * Kernel timing for benchmarks.  While enabled, every operator call (also inside
+ * the block calls) is bracketed by HIP events recorded on its launch stream.
+ * msd_profile_read waits for the recorded events and returns, per class
+ * {0 forward, 1 backward_x incl. the mask, 2 backward_k/bias}, the summed elapsed
+ * milliseconds and the number of calls since msd_profile_enable(1).  Not thread-safe;
+ * no counterpart in the reference.
+ */
+int msd_profile_enable(int on);
+int msd_profile_read(double *ms, int64_t *calls);
+
 #ifdef __cplusplus
 }
 #endif

@@ -40,6 +40,14 @@ PROTOTYPES = {
     "msd_conv_relu_backward_kb": (_c_int, _HEAD + _VIEW + _VIEW + _VIEW + [_ptr, _ptr] + _WS + [_ptr]),
     "msd_conv_backward_kb": (_c_int, _HEAD + _VIEW + _VIEW + [_ptr, _ptr] + _WS + [_ptr]),
     "msd_relu_mask_gradient": (_c_int, [_c_int, _c_int, _c_i64, _c_i64, _i64p] + _VIEW + _VIEW + [_ptr]),
+    "msd_block_workspace_bytes": (_c_i64, [_c_int, _c_int, _c_i64, _c_i64, _c_int, _i64p, _i64p]),
+    "msd_block_forward": (_c_int, [_c_int, _c_int, _c_i64, _c_i64, _c_int, _i64p, _i64p, _i64p] + _VIEW
+                          + [ctypes.POINTER(ctypes.c_void_p), _ptr, _ptr]),
+    "msd_block_backward": (_c_int, [_c_int, _c_int, _c_i64, _c_i64, _c_int, _i64p, _i64p, _i64p] + _VIEW + _VIEW
+                           + [ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ctypes.c_void_p), _ptr, _c_int]
+                           + _WS + [_ptr]),
+    "msd_profile_enable": (_c_int, [_c_int]),
+    "msd_profile_read": (_c_int, [ctypes.POINTER(ctypes.c_double), _i64p]),
 }
 
 _lib = None

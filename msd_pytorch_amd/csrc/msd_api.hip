@@ -7,6 +7,8 @@
 #include <cstdarg>
 #include <cstdio>
 #include <string>
+#include <utility>
+#include <vector>
 
 namespace msd {
 const char *const kKnobNames[kKnobCount] = {
@@ -27,6 +29,46 @@ int g_kernel_path = 0;
 
 template <typename T> struct is_f32 { static constexpr bool value = false; };
 template <> struct is_f32<float> { static constexpr bool value = true; };
+
+// Optional per-class kernel timing with HIP events recorded on the launch stream
+// (msd_profile_* in the C ABI).  Classes: 0 forward, 1 backward_x (+ mask), 2 backward_k/bias.
+struct Profile {
+    bool on = false;
+    std::vector<hipEvent_t> pool;                           // reused across calls
+    size_t used = 0;
+    std::vector<std::pair<size_t, size_t>> spans[3];        // (start, stop) indices into pool
+    hipEvent_t take()
+    {
+        if (used == pool.size()) {
+            hipEvent_t e;
+            if (hipEventCreate(&e) != hipSuccess) return nullptr;
+            pool.push_back(e);
+        }
+        return pool[used++];
+    }
+} g_profile;
+
+// Records an event pair around the launches made during its lifetime.
+struct ProfileScope {
+    int cls;
+    hipStream_t s;
+    size_t start = 0;
+    bool active;
+    ProfileScope(int cls_, hipStream_t s_) : cls(cls_), s(s_), active(g_profile.on)
+    {
+        if (!active) return;
+        start = g_profile.used;
+        hipEvent_t e = g_profile.take();
+        if (!e || hipEventRecord(e, s) != hipSuccess) active = false;
+    }
+    ~ProfileScope()
+    {
+        if (!active) return;
+        const size_t stop = g_profile.used;
+        hipEvent_t e = g_profile.take();
+        if (e && hipEventRecord(e, s) == hipSuccess) g_profile.spans[cls].push_back({start, stop});
+    }
+};
 
 int fail(int code, const char *fmt, ...)
 {
@@ -121,6 +163,7 @@ int forward_t(const char *fn, bool relu, const msd::Geom &g, int ndim, const voi
     MSD_TRY(make_view(fn, "output", ndim, output, os, &y));
     if (!kernel) return fail(MSD_ERR_INVALID, "%s: kernel is NULL", fn);
     if (!bias) return fail(MSD_ERR_INVALID, "%s: bias is NULL", fn);
+    ProfileScope scope(0, s);
     hipError_t e;
     if constexpr (is_f32<T>::value) {
         if (g_kernel_path == 0 && msd::fast_forward_supported(g, x, y))
@@ -148,7 +191,7 @@ int forward(const char *fn, bool relu, int dtype, int ndim, int64_t batch, int64
 template <typename T>
 int backward_x_t(const char *fn, bool relu, const msd::Geom &g, int ndim, const void *output, const int64_t *os,
                  const void *grad_output, const int64_t *gs, const void *kernel, void *grad_input,
-                 const int64_t *xs, hipStream_t s)
+                 const int64_t *xs, hipStream_t s, int mask_from, const void *act, const int64_t *as, bool *masked)
 {
     msd::View<const T> o{nullptr, 0, 0, 0, 0, 0}, gy;
     msd::View<T> gx;
@@ -156,11 +199,24 @@ int backward_x_t(const char *fn, bool relu, const msd::Geom &g, int ndim, const 
     MSD_TRY(make_view(fn, "grad_output", ndim, grad_output, gs, &gy));
     MSD_TRY(make_view(fn, "grad_input", ndim, grad_input, xs, &gx));
     if (!kernel) return fail(MSD_ERR_INVALID, "%s: kernel is NULL", fn);
+    ProfileScope scope(1, s);
     hipError_t e;
     if constexpr (is_f32<T>::value) {
-        if (g_kernel_path == 0 && msd::fast_backward_x_supported(g, relu, o, gy, gx))
-            e = msd::fast_backward_x(g, relu, o, gy, (const float *)kernel, gx, s);
-        else
+        if (g_kernel_path == 0 && msd::fast_backward_x_supported(g, relu, o, gy, gx)) {
+            msd::PostMask pm{g.C, {nullptr, 0, 0, 0, 0, 0}};
+            if (act && as && as[ndim + 1] == 1) {
+                // the activation view must allow the same aligned V-wide loads as grad_input
+                msd::View<const float> av;
+                MSD_TRY(make_view(fn, "activation", ndim, act, as, &av));
+                const bool same_layout = av.sb == gx.sb && av.sc == gx.sc && av.sz == gx.sz && av.sy == gx.sy &&
+                                         reinterpret_cast<uintptr_t>(av.p) % 16 == reinterpret_cast<uintptr_t>(gx.p) % 16;
+                if (same_layout) {
+                    pm = msd::PostMask{mask_from, av};
+                    if (masked) *masked = true;
+                }
+            }
+            e = msd::fast_backward_x(g, relu, o, gy, (const float *)kernel, gx, pm, s);
+        } else
             e = msd::generic_backward_x<T>(g, relu, o, gy, (const T *)kernel, gx, s);
     } else {
         e = msd::generic_backward_x<T>(g, relu, o, gy, (const T *)kernel, gx, s);
@@ -170,15 +226,19 @@ int backward_x_t(const char *fn, bool relu, const msd::Geom &g, int ndim, const 
 
 int backward_x(const char *fn, bool relu, int dtype, int ndim, int64_t batch, int64_t c_in, int64_t c_out,
                const int64_t *spatial, int dilation, const void *output, const int64_t *os, const void *grad_output,
-               const int64_t *gs, const void *kernel, void *grad_input, const int64_t *xs, void *stream)
+               const int64_t *gs, const void *kernel, void *grad_input, const int64_t *xs, void *stream,
+               int mask_from = 0, const void *act = nullptr, const int64_t *as = nullptr, bool *masked = nullptr)
 {
+    // act/as/mask_from: optional ReLU mask applied to grad_input channels >= mask_from on the
+    // way out (dense block only); *masked reports whether the kernel that ran did it.
     msd::Geom g;
     MSD_TRY(make_geom(fn, dtype, ndim, batch, c_in, c_out, spatial, dilation, true, &g));
     if (c_in <= 0) return fail(MSD_ERR_INVALID, "%s: c_in must be positive", fn);
+    if (masked) *masked = false;
     return dtype == MSD_F32 ? backward_x_t<float>(fn, relu, g, ndim, output, os, grad_output, gs, kernel, grad_input,
-                                                  xs, (hipStream_t)stream)
+                                                  xs, (hipStream_t)stream, mask_from, act, as, masked)
                             : backward_x_t<double>(fn, relu, g, ndim, output, os, grad_output, gs, kernel, grad_input,
-                                                   xs, (hipStream_t)stream);
+                                                   xs, (hipStream_t)stream, mask_from, act, as, masked);
 }
 
 template <typename T>
@@ -192,6 +252,7 @@ int backward_kb_t(const char *fn, bool relu, const msd::Geom &g, int ndim, const
     if (grad_kernel) MSD_TRY(make_view(fn, "input", ndim, input, xs, &x));
     if (!grad_kernel && !grad_bias) return fail(MSD_ERR_INVALID, "%s: no gradient buffer given", fn);
     MSD_TRY(check_workspace(fn, g, sizeof(T), ws, ws_bytes));
+    ProfileScope scope(2, s);
     hipError_t e;
     if constexpr (is_f32<T>::value) {
         if (g_kernel_path == 0 && grad_kernel && msd::fast_backward_kb_supported(g, relu, o, gy, x))
@@ -343,6 +404,7 @@ int msd_relu_mask_gradient(int dtype, int ndim, int64_t batch, int64_t c_out, co
     const char *fn = "relu_mask_gradient";
     msd::Geom g;
     MSD_TRY(make_geom(fn, dtype, ndim, batch, 0, c_out, spatial, 1, false, &g));
+    ProfileScope scope(1, (hipStream_t)stream);
     if (dtype == MSD_F32) {
         msd::View<const float> o;
         msd::View<float> gy;
@@ -368,6 +430,156 @@ int msd_conv_relu_backward_kb(int dtype, int ndim, int64_t batch, int64_t c_in, 
     return backward_kb("conv_relu_backward_kb", true, true, dtype, ndim, batch, c_in, c_out, spatial, dilation, output,
                        output_strides, grad_output, grad_output_strides, input, input_strides, grad_kernel, grad_bias,
                        workspace, workspace_bytes, stream);
+}
+
+
+// ---------------------------------------------------------------------------
+// Dense block: the layer loops of msd_block.py:40-58 (forward) and :89-130
+// (backward) as one native call each, so a training step costs two library calls
+// per block instead of four Python-level operator calls per layer.
+// ---------------------------------------------------------------------------
+
+namespace {
+
+struct BlockArgs {
+    int dtype, ndim, depth;
+    int64_t batch, c_in, c_total;
+    const int64_t *widths, *spatial, *dilations;
+    size_t elem;
+};
+
+int check_block(const char *fn, int dtype, int ndim, int64_t batch, int64_t c_in, int depth, const int64_t *widths,
+                const int64_t *spatial, const int64_t *dilations, const void *stack, const int64_t *stack_strides,
+                const void *const *weights, BlockArgs *a)
+{
+    if (dtype != MSD_F32 && dtype != MSD_F64) return fail(MSD_ERR_INVALID, "%s: dtype must be MSD_F32 or MSD_F64", fn);
+    if (ndim != 2 && ndim != 3) return fail(MSD_ERR_INVALID, "%s: expected 2 or 3 spatial dimensions, got %d", fn, ndim);
+    if (depth <= 0 || c_in <= 0 || batch <= 0) return fail(MSD_ERR_INVALID, "%s: depth, c_in and batch must be positive", fn);
+    if (!widths || !spatial || !dilations || !stack || !stack_strides || !weights)
+        return fail(MSD_ERR_INVALID, "%s: NULL argument", fn);
+    int64_t total = c_in;
+    for (int i = 0; i < depth; i++) {
+        if (widths[i] <= 0) return fail(MSD_ERR_INVALID, "%s: layer widths must be positive", fn);
+        if (!weights[i]) return fail(MSD_ERR_INVALID, "%s: weights[%d] is NULL", fn, i);
+        if (dilations[i] <= 0) return fail(MSD_ERR_INVALID, "%s: Dilation must be 1 or greater", fn);
+        for (int d = 0; d < ndim; d++)
+            if (dilations[i] > spatial[d])
+                return fail(MSD_ERR_INVALID, "%s: Dilation cannot be greater than size of image.", fn);
+        total += widths[i];
+    }
+    *a = BlockArgs{dtype, ndim, depth, batch, c_in, total, widths, spatial, dilations, dtype == MSD_F32 ? 4u : 8u};
+    return MSD_OK;
+}
+
+}  // namespace
+
+int64_t msd_block_workspace_bytes(int dtype, int ndim, int64_t batch, int64_t c_in, int depth, const int64_t *widths,
+                                  const int64_t *spatial)
+{
+    if (!widths || depth <= 0) return -1;
+    int64_t total = c_in, wmax = 0, need = 0;
+    for (int i = 0; i < depth; i++) {
+        if (widths[i] <= 0) return -1;
+        wmax = widths[i] > wmax ? widths[i] : wmax;
+        const int64_t n = msd_workspace_bytes(dtype, ndim, batch, total, widths[i], spatial);
+        if (n < 0) return -1;
+        need = n > need ? n : need;
+        total += widths[i];
+    }
+    return need;
+}
+
+int msd_block_forward(int dtype, int ndim, int64_t batch, int64_t c_in, int depth, const int64_t *widths,
+                      const int64_t *spatial, const int64_t *dilations, void *stack, const int64_t *stack_strides,
+                      const void *const *weights, const void *bias, void *stream)
+{
+    const char *fn = "block_forward";
+    BlockArgs a;
+    MSD_TRY(check_block(fn, dtype, ndim, batch, c_in, depth, widths, spatial, dilations, stack, stack_strides,
+                        weights, &a));
+    if (!bias) return fail(MSD_ERR_INVALID, "%s: bias is NULL", fn);
+    int64_t first = c_in, b0 = 0;
+    for (int i = 0; i < depth; i++) {
+        char *out = (char *)stack + first * stack_strides[1] * a.elem;
+        MSD_TRY(forward("conv_relu_forward", true, dtype, ndim, batch, first, widths[i], spatial, (int)dilations[i],
+                        stack, stack_strides, weights[i], (const char *)bias + b0 * a.elem, out, stack_strides,
+                        stream));
+        first += widths[i];
+        b0 += widths[i];
+    }
+    return MSD_OK;
+}
+
+int msd_block_backward(int dtype, int ndim, int64_t batch, int64_t c_in, int depth, const int64_t *widths,
+                       const int64_t *spatial, const int64_t *dilations, const void *stack,
+                       const int64_t *stack_strides, void *grads, const int64_t *grads_strides,
+                       const void *const *weights, void *const *grad_weights, void *grad_bias, int need_input_grad,
+                       void *workspace, int64_t workspace_bytes, void *stream)
+{
+    const char *fn = "block_backward";
+    BlockArgs a;
+    MSD_TRY(check_block(fn, dtype, ndim, batch, c_in, depth, widths, spatial, dilations, stack, stack_strides,
+                        weights, &a));
+    if (!grads || !grads_strides || !grad_weights) return fail(MSD_ERR_INVALID, "%s: NULL argument", fn);
+    int64_t last = a.c_total, b1 = a.c_total - c_in;
+    bool masked = false;   // the mask of the current layer was already applied by the previous backward_x
+    for (int i = depth - 1; i >= 0; i--) {
+        const int64_t w = widths[i], first = last - w, b0 = b1 - w;
+        const char *out_i = (const char *)stack + first * stack_strides[1] * a.elem;
+        char *gout_i = (char *)grads + first * grads_strides[1] * a.elem;
+        // The layer's slice of the private gradient stack is not read again after this
+        // iteration: its ReLU mask is applied once, in place, and the plain operators do
+        // the rest.  Where the specialised backward_x runs, the mask of layer i-1 rides
+        // on layer i's update of those channels (their last one); otherwise, and for
+        // the top layer, a separate pass applies it.
+        if (!masked)
+            MSD_TRY(msd_relu_mask_gradient(dtype, ndim, batch, w, spatial, out_i, stack_strides, gout_i,
+                                           grads_strides, stream));
+        masked = false;
+        if (i > 0 || need_input_grad)
+            MSD_TRY(backward_x("conv_backward_x", false, dtype, ndim, batch, first, w, spatial, (int)dilations[i],
+                               nullptr, nullptr, gout_i, grads_strides, weights[i], grads, grads_strides, stream,
+                               i > 0 ? (int)(first - widths[i - 1]) : (int)first, i > 0 ? stack : nullptr,
+                               stack_strides, &masked));
+        void *gb = grad_bias ? (char *)grad_bias + b0 * a.elem : nullptr;
+        if (grad_weights[i])
+            MSD_TRY(backward_kb("conv_backward_kb", false, true, dtype, ndim, batch, first, w, spatial,
+                                (int)dilations[i], nullptr, nullptr, gout_i, grads_strides, stack, stack_strides,
+                                grad_weights[i], gb, workspace, workspace_bytes, stream));
+        else if (gb)
+            MSD_TRY(backward_kb("conv_backward_bias", false, false, dtype, ndim, batch, 0, w, spatial, 1, nullptr,
+                                nullptr, gout_i, grads_strides, nullptr, nullptr, nullptr, gb, workspace,
+                                workspace_bytes, stream));
+        last = first;
+        b1 = b0;
+    }
+    return MSD_OK;
+}
+
+int msd_profile_enable(int on)
+{
+    g_profile.on = on != 0;
+    g_profile.used = 0;
+    for (auto &v : g_profile.spans) v.clear();
+    return MSD_OK;
+}
+
+int msd_profile_read(double *ms, int64_t *calls)
+{
+    if (!ms || !calls) return fail(MSD_ERR_INVALID, "msd_profile_read: NULL argument");
+    for (int c = 0; c < 3; c++) {
+        double total = 0;
+        for (const auto &sp : g_profile.spans[c]) {
+            hipError_t e = hipEventSynchronize(g_profile.pool[sp.second]);
+            float t = 0;
+            if (e == hipSuccess) e = hipEventElapsedTime(&t, g_profile.pool[sp.first], g_profile.pool[sp.second]);
+            if (e != hipSuccess) return hip_fail("msd_profile_read", e);
+            total += t;
+        }
+        ms[c] = total;
+        calls[c] = (int64_t)g_profile.spans[c].size();
+    }
+    return MSD_OK;
 }
 
 }  // extern "C"

@@ -10,9 +10,9 @@ bool fast_backward_x_supported_2d(const Geom &g, bool relu, const View<const flo
 }
 
 hipError_t fast_backward_x_2d(const Geom &g, bool relu, const View<const float> &out, const View<const float> &gy,
-                               const float *k, const View<float> &gx, hipStream_t s)
+                               const float *k, const View<float> &gx, const PostMask &pm, hipStream_t s)
 {
-    return bwdx::fast_backward_x_nd<2>(g, relu, out, gy, k, gx, s);
+    return bwdx::fast_backward_x_nd<2>(g, relu, out, gy, k, gx, pm, s);
 }
 
 }  // namespace msd

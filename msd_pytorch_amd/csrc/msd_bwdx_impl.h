@@ -16,7 +16,8 @@ namespace bwdx {
 
 template <int NDIM, bool RELU, int WOUT, int V, int U, int MAXT>
 __global__ __launch_bounds__(MAXT) void bwdx_rows(Geom g, RowTeams rt, int cch, int remap, View<const float> out,
-                                                  View<const float> gy, const float *__restrict__ k, View<float> gx)
+                                                  View<const float> gy, const float *__restrict__ k, View<float> gx,
+                                                  PostMask pm)
 {
     extern __shared__ float lds[];
     constexpr int K = Taps<NDIM>::K, NPQ = RowTaps<NDIM>::NPQ;
@@ -78,6 +79,16 @@ __global__ __launch_bounds__(MAXT) void bwdx_rows(Geom g, RowTeams rt, int cch, 
             }
 #pragma unroll
             for (int i = 0; i < V; i++) cur[u][i] += s[i];
+            // channels from pm.from on are outputs of the layer below: their gradient is
+            // complete with this update, so its ReLU mask is applied on the way out
+            if (cu[u] >= pm.from) {
+                float a[V];
+                load_vec<V>(pm.act.p + (int64_t)b * pm.act.sb + (int64_t)cu[u] * pm.act.sc + (int64_t)z * pm.act.sz +
+                                (int64_t)y * pm.act.sy + x0,
+                            a);
+#pragma unroll
+                for (int i = 0; i < V; i++) cur[u][i] = 0.f < a[i] ? cur[u][i] : 0.f;
+            }
         }
 #pragma unroll
         for (int u = 0; u < U; u++)
@@ -89,7 +100,7 @@ constexpr size_t kMaxLds = 64 * 1024;
 
 template <int NDIM, bool RELU, int WOUT, int V, int U>
 hipError_t launch(const Geom &g, const View<const float> &out, const View<const float> &gy, const float *k,
-                  const View<float> &gx, hipStream_t s)
+                  const View<float> &gx, const PostMask &pm, hipStream_t s)
 {
     RowTeams rt;
     make_row_teams(g, V, &rt);
@@ -106,11 +117,11 @@ hipError_t launch(const Geom &g, const View<const float> &out, const View<const 
     const dim3 grid(remap ? xcd_grid(nb) : nb, g.B, chunks);
     if (rt.lpr * rt.rpw <= 256) {
         hipLaunchKernelGGL((bwdx_rows<NDIM, RELU, WOUT, V, U, 256>), grid, dim3(rt.lpr * rt.rpw), lds,
-                           s, g, rt, cch, remap, out, gy, k, gx);
+                           s, g, rt, cch, remap, out, gy, k, gx, pm);
     } else if constexpr (V == 4) {
         // rows longer than 1024 voxels: up to 1024 lanes per workgroup
         hipLaunchKernelGGL((bwdx_rows<NDIM, RELU, WOUT, V, U, 1024>), grid, dim3(rt.lpr * rt.rpw), lds,
-                           s, g, rt, cch, remap, out, gy, k, gx);
+                           s, g, rt, cch, remap, out, gy, k, gx, pm);
     } else {
         return hipErrorInvalidConfiguration;   // excluded by fits()
     }
@@ -119,11 +130,11 @@ hipError_t launch(const Geom &g, const View<const float> &out, const View<const 
 
 template <int NDIM, bool RELU, int WOUT, int V>
 hipError_t pick_unroll(const Geom &g, const View<const float> &out, const View<const float> &gy, const float *k,
-                       const View<float> &gx, hipStream_t s)
+                       const View<float> &gx, const PostMask &pm, hipStream_t s)
 {
     const int u = knob(NDIM == 3 ? kKnobBwdxUnroll3d : kKnobBwdxUnroll2d, 2);
-    if (u <= 2) return launch<NDIM, RELU, WOUT, V, 2>(g, out, gy, k, gx, s);
-    return launch<NDIM, RELU, WOUT, V, 4>(g, out, gy, k, gx, s);
+    if (u <= 2) return launch<NDIM, RELU, WOUT, V, 2>(g, out, gy, k, gx, pm, s);
+    return launch<NDIM, RELU, WOUT, V, 4>(g, out, gy, k, gx, pm, s);
 }
 
 // Row fits a workgroup and its staged rows fit the LDS budget.
@@ -153,23 +164,23 @@ int choose_vec(const Geom &g, bool relu, int wout, int vmax, const View<const fl
 
 template <int NDIM, bool RELU, int WOUT>
 hipError_t pick_vec(const Geom &g, const View<const float> &out, const View<const float> &gy, const float *k,
-                    const View<float> &gx, hipStream_t s)
+                    const View<float> &gx, const PostMask &pm, hipStream_t s)
 {
     // registers: the gathered gradient takes WOUT * K * V of them
     const int vmax = knob(NDIM == 3 ? kKnobBwdxVec3d : kKnobBwdxVec2d, NDIM == 3 ? 1 : 4);
     int v = choose_vec<NDIM>(g, RELU, WOUT, vmax, out, gy, gx);
     if (v == 0) v = choose_vec<NDIM>(g, RELU, WOUT, 4, out, gy, gx);
-    if (v == 4) return pick_unroll<NDIM, RELU, WOUT, 4>(g, out, gy, k, gx, s);
-    if (v == 2) return pick_unroll<NDIM, RELU, WOUT, 2>(g, out, gy, k, gx, s);
-    if (v == 1) return pick_unroll<NDIM, RELU, WOUT, 1>(g, out, gy, k, gx, s);
+    if (v == 4) return pick_unroll<NDIM, RELU, WOUT, 4>(g, out, gy, k, gx, pm, s);
+    if (v == 2) return pick_unroll<NDIM, RELU, WOUT, 2>(g, out, gy, k, gx, pm, s);
+    if (v == 1) return pick_unroll<NDIM, RELU, WOUT, 1>(g, out, gy, k, gx, pm, s);
     return hipErrorInvalidConfiguration;   // callers check fast_backward_x_supported first
 }
 
 template <int NDIM, bool RELU>
 hipError_t pick_wout(const Geom &g, const View<const float> &out, const View<const float> &gy, const float *k,
-                     const View<float> &gx, hipStream_t s)
+                     const View<float> &gx, const PostMask &pm, hipStream_t s)
 {
-    return g.Wd == 1 ? pick_vec<NDIM, RELU, 1>(g, out, gy, k, gx, s) : pick_vec<NDIM, RELU, 2>(g, out, gy, k, gx, s);
+    return g.Wd == 1 ? pick_vec<NDIM, RELU, 1>(g, out, gy, k, gx, pm, s) : pick_vec<NDIM, RELU, 2>(g, out, gy, k, gx, pm, s);
 }
 
 template <int NDIM>
@@ -183,9 +194,9 @@ bool fast_backward_x_supported_nd(const Geom &g, bool relu, const View<const flo
 
 template <int NDIM>
 hipError_t fast_backward_x_nd(const Geom &g, bool relu, const View<const float> &out, const View<const float> &gy,
-                              const float *k, const View<float> &gx, hipStream_t s)
+                              const float *k, const View<float> &gx, const PostMask &pm, hipStream_t s)
 {
-    return relu ? pick_wout<NDIM, true>(g, out, gy, k, gx, s) : pick_wout<NDIM, false>(g, out, gy, k, gx, s);
+    return relu ? pick_wout<NDIM, true>(g, out, gy, k, gx, pm, s) : pick_wout<NDIM, false>(g, out, gy, k, gx, pm, s);
 }
 
 }  // namespace bwdx

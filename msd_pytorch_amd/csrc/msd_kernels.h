@@ -46,14 +46,23 @@ extern const char *const kKnobNames[kKnobCount];
 extern int g_knobs[kKnobCount];
 
 // Specialised fp32 kernels (unit x-stride, one or two output channels).
+// Optional epilogue of the specialised backward_x: grad_input channels >= from are
+// multiplied by [0 < act] after the update (act is viewed like grad_input).  The
+// dense block uses it to apply the ReLU mask of the layer below while its gradient
+// is written for the last time.  from >= C disables it.
+struct PostMask {
+    int from;
+    View<const float> act;
+};
+
 bool fast_backward_x_supported_2d(const Geom &g, bool relu, const View<const float> &out,
                                   const View<const float> &gy, const View<float> &gx);
 bool fast_backward_x_supported_3d(const Geom &g, bool relu, const View<const float> &out,
                                   const View<const float> &gy, const View<float> &gx);
 hipError_t fast_backward_x_2d(const Geom &g, bool relu, const View<const float> &out, const View<const float> &gy,
-                              const float *k, const View<float> &gx, hipStream_t s);
+                              const float *k, const View<float> &gx, const PostMask &pm, hipStream_t s);
 hipError_t fast_backward_x_3d(const Geom &g, bool relu, const View<const float> &out, const View<const float> &gy,
-                              const float *k, const View<float> &gx, hipStream_t s);
+                              const float *k, const View<float> &gx, const PostMask &pm, hipStream_t s);
 
 inline bool fast_backward_x_supported(const Geom &g, bool relu, const View<const float> &out,
                                       const View<const float> &gy, const View<float> &gx)
@@ -62,9 +71,10 @@ inline bool fast_backward_x_supported(const Geom &g, bool relu, const View<const
                        : fast_backward_x_supported_2d(g, relu, out, gy, gx);
 }
 inline hipError_t fast_backward_x(const Geom &g, bool relu, const View<const float> &out, const View<const float> &gy,
-                                  const float *k, const View<float> &gx, hipStream_t s)
+                                  const float *k, const View<float> &gx, const PostMask &pm, hipStream_t s)
 {
-    return g.ndim == 3 ? fast_backward_x_3d(g, relu, out, gy, k, gx, s) : fast_backward_x_2d(g, relu, out, gy, k, gx, s);
+    return g.ndim == 3 ? fast_backward_x_3d(g, relu, out, gy, k, gx, pm, s)
+                       : fast_backward_x_2d(g, relu, out, gy, k, gx, pm, s);
 }
 
 bool fast_forward_supported_2d(const Geom &g, const View<const float> &x, const View<float> &out);

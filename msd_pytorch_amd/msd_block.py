@@ -29,12 +29,8 @@ class MSDBlockFunction(torch.autograd.Function):
         stack = input.new_empty(input.shape[0], c_in + sum(widths), *input.shape[2:])
         stack[:, :c_in] = input
 
-        first, b0 = c_in, 0
-        for weight, width, dilation in zip(weights, widths, dilations):
-            cc.conv_relu_forward(stack[:, :first], weight, bias[b0:b0 + width],
-                                 stack[:, first:first + width], dilation)
-            first += width
-            b0 += width
+        # the layer loop of msd_block.py:40-58 runs inside the native library
+        cc.block_forward(stack, c_in, list(dilations), bias, list(weights))
 
         ctx.dilations = tuple(dilations)
         ctx.save_for_backward(bias, stack, *weights)
@@ -50,34 +46,27 @@ class MSDBlockFunction(torch.autograd.Function):
         # Working copy of the incoming gradient: layer idx adds its input
         # gradient to channels [0, first), which later iterations consume.
         grads = grad_output.clone()
-        grad_bias = torch.zeros_like(bias)
+        grad_bias = torch.zeros_like(bias) if need_bias else None
         grad_weights = [None] * len(weights)
 
-        last, b1 = stack.shape[1], bias.shape[0]
-        for idx in reversed(range(len(weights))):
-            weight = weights[idx]
-            width = weight.shape[0]
-            first, b0 = last - width, b1 - width
-            out_i, gout_i = stack[:, first:last], grads[:, first:last]
-            dilation = ctx.dilations[idx]
-
-            # `grads` is private to this call and the layer's slice is not read again
-            # afterwards, so the ReLU mask is applied to it once, in place, and the
-            # plain operators do the rest (the reference masks on the fly in each of
-            # conv_relu_backward_x / _k / _bias, msd_block.py:107-126).
-            cc.relu_mask_gradient(out_i, gout_i)
-            if idx > 0 or need_input:
-                cc.conv_backward_x(gout_i, weight, grads[:, :first], dilation)
+        # The reverse layer loop of msd_block.py:89-130 runs inside the native library.
+        # Per layer it masks the layer's slice of `grads` once in place (the slice is
+        # private to this call and not read again afterwards) and then applies the
+        # plain backward operators; the reference masks on the fly in each of
+        # conv_relu_backward_x / _k / _bias.
+        # one zero-filled buffer for all weight gradients (one fill instead of one per layer)
+        wanted = [w for w, need in zip(weights, need_weights) if need]
+        flat = stack.new_zeros(sum(w.numel() for w in wanted))
+        offset = 0
+        for idx, weight in enumerate(weights):
             if need_weights[idx]:
-                grad_weights[idx] = torch.zeros_like(weight)
-                cc.conv_backward_kb(gout_i, stack[:, :first], grad_weights[idx],
-                                    grad_bias[b0:b1] if need_bias else None, dilation)
-            elif need_bias:
-                cc.conv_backward_bias(gout_i, grad_bias[b0:b1])
-            last, b1 = first, b0
+                grad_weights[idx] = flat[offset:offset + weight.numel()].view_as(weight)
+                offset += weight.numel()
+        cc.block_backward(stack, grads, weights[0].shape[1], list(ctx.dilations), list(weights), grad_weights,
+                          grad_bias if need_bias else None, bool(need_input))
 
         grad_input = grads[:, :weights[0].shape[1]] if need_input else None
-        return (grad_input, None, grad_bias if need_bias else None, *grad_weights)
+        return (grad_input, None, grad_bias, *grad_weights)
 
 
 msd_block = MSDBlockFunction.apply

@@ -307,3 +307,83 @@ def conv_relu_backward_bias(output, grad_output, grad_bias, block_size=None):
     """grad_bias += grad_output summed where output > 0 (msd_custom_convolutions.cpp:318-338)."""
     _backward_bias("conv_relu_backward_bias", "msd_conv_relu_backward_bias", output, grad_output, grad_bias,
                    block_size)
+
+
+# ---------------------------------------------------------------------------
+# Dense block as one native call per direction (not part of the reference's
+# module: there the loops of msd_block.py:40-58 and :89-130 run in Python).
+# ---------------------------------------------------------------------------
+
+def _check_block(fn, stack, c_in, dilations, bias, weights):
+    named = [("stack", stack), ("bias", bias)] + [(f"weight{i}", w) for i, w in enumerate(weights)]
+    _check_same_gpu(fn, named)
+    _check_same_type(fn, named)
+    if stack.dim() not in (4, 5):
+        _fail(fn, f"expected a 4- or 5-dimensional stack, got {stack.dim()} dimensions")
+    if len(dilations) != len(weights):
+        _fail(fn, "number of weights does not match depth")
+    channels = c_in
+    for i, (w, d) in enumerate(zip(weights, dilations)):
+        _check_kernel(fn, w)
+        _check_dim(fn, f"weight{i}", w, stack.dim())
+        if w.shape[1] != channels:
+            _fail(fn, "Kernel shape does not match input channels. ")
+        _check_dilation(fn, stack, d)
+        channels += w.shape[0]
+    if channels != stack.shape[1]:
+        _fail(fn, "Kernel shape does not match output channels. ")
+    _check_dim(fn, "bias", bias, 1)
+    if bias.shape[0] != channels - c_in:
+        _fail(fn, "Bias shape does not match output channels. ")
+
+
+def _block_head(stack, c_in, dilations, weights):
+    widths = _native.i64_array([w.shape[0] for w in weights])
+    return (_DTYPES[stack.dtype], stack.dim() - 2, stack.shape[0], c_in, len(weights), widths,
+            _native.i64_array(tuple(stack.shape[2:])), _native.i64_array(list(dilations)))
+
+
+def _ptr_array(tensors):
+    return (ctypes.c_void_p * len(tensors))(*[t.data_ptr() if t is not None else None for t in tensors])
+
+
+def block_forward(stack, c_in, dilations, bias, weights):
+    """Fill channels [c_in, end) of ``stack`` layer by layer; channels [0, c_in)
+    hold the block's input.  Layer i: conv_relu_forward(stack[:, :C_i], weights[i],
+    bias slice, stack[:, C_i:C_i + width_i], dilations[i])."""
+    fn = "block_forward"
+    _check_block(fn, stack, c_in, dilations, bias, weights)
+    bias = bias.contiguous()
+    _call("msd_block_forward", stack.device, *_block_head(stack, c_in, dilations, weights), *_view(stack),
+          _ptr_array(weights), ctypes.c_void_p(bias.data_ptr()), _stream(stack))
+
+
+def block_backward(stack, grads, c_in, dilations, weights, grad_weights, grad_bias, need_input_grad):
+    """Backward of the whole block.  ``grads`` holds dL/dstack and is overwritten
+    (it is the caller's private working copy); afterwards grads[:, :c_in] is
+    dL/dinput.  ``grad_weights[i]`` (zero-filled, or None to skip) and ``grad_bias``
+    (zero-filled, or None) are accumulated into."""
+    fn = "block_backward"
+    _check_block(fn, stack, c_in, dilations, torch.empty(stack.shape[1] - c_in, dtype=stack.dtype,
+                                                          device=stack.device) if grad_bias is None else grad_bias,
+                 weights)
+    named = [("stack", stack), ("grads", grads)] + [(f"grad_weight{i}", g) for i, g in enumerate(grad_weights)
+                                                    if g is not None]
+    _check_same_gpu(fn, named)
+    _check_same_type(fn, named)
+    if tuple(grads.shape) != tuple(stack.shape):
+        _fail(fn, "Input shape does not match output shape. ")
+    for g, w in zip(grad_weights, weights):
+        if g is not None and (tuple(g.shape) != tuple(w.shape) or not g.is_contiguous()):
+            _fail(fn, "grad_weights must be contiguous and shaped like the weights")
+    if grad_bias is not None and not grad_bias.is_contiguous():
+        _fail(fn, "Expected grad_bias to be contiguous")
+    head = _block_head(stack, c_in, dilations, weights)
+    lib = _native.load()
+    need = lib.msd_block_workspace_bytes(head[0], head[1], head[2], c_in, head[4], head[5], head[6])
+    if need < 0:
+        _fail(fn, "invalid block geometry")
+    ws = torch.empty(max(int(need), 8), dtype=torch.uint8, device=stack.device)
+    _call("msd_block_backward", stack.device, *head, *_view(stack), *_view(grads), _ptr_array(weights),
+          _ptr_array(grad_weights), ctypes.c_void_p(grad_bias.data_ptr() if grad_bias is not None else 0),
+          1 if need_input_grad else 0, ctypes.c_void_p(ws.data_ptr()), int(need), _stream(stack))

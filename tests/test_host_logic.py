@@ -39,6 +39,30 @@ def oracle_ops(monkeypatch):
             oracle.conv_backward_bias(grad_output, grad_bias)
     monkeypatch.setattr(cc, "conv_backward_kb", plain_kb)
 
+    def block_forward(stack, c_in, dilations, bias, weights):
+        first, b0 = c_in, 0
+        for w, d in zip(weights, dilations):
+            n = w.shape[0]
+            oracle.conv_relu_forward(stack[:, :first], w, bias[b0:b0 + n], stack[:, first:first + n], d)
+            first, b0 = first + n, b0 + n
+    monkeypatch.setattr(cc, "block_forward", block_forward)
+
+    def block_backward(stack, grads, c_in, dilations, weights, grad_weights, grad_bias, need_input_grad):
+        last = stack.shape[1]
+        b1 = last - c_in
+        for idx in reversed(range(len(weights))):
+            n = weights[idx].shape[0]
+            first, b0 = last - n, b1 - n
+            out_i, gout_i = stack[:, first:last], grads[:, first:last]
+            if idx > 0 or need_input_grad:
+                oracle.conv_relu_backward_x(out_i, gout_i, weights[idx], grads[:, :first], dilations[idx])
+            if grad_weights[idx] is not None:
+                oracle.conv_relu_backward_k(out_i, gout_i, stack[:, :first], grad_weights[idx], dilations[idx])
+            if grad_bias is not None:
+                oracle.conv_relu_backward_bias(out_i, gout_i, grad_bias[b0:b1])
+            last, b1 = first, b0
+    monkeypatch.setattr(cc, "block_backward", block_backward)
+
     def mask(output, grad_output):
         grad_output.mul_((output > 0).to(grad_output.dtype))
     monkeypatch.setattr(cc, "relu_mask_gradient", mask)
