@@ -161,6 +161,8 @@ def main():
     ap.add_argument("--workload", default="C", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-timing", action="store_true")
+    ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
+                    help="launch-shape knob passed to msd_set_tuning (repeatable)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run one 1 GiB device copy first (reference dispatch for scaling rocprof byte counters)")
     args = ap.parse_args()
@@ -172,6 +174,11 @@ def main():
     lib = _native.load()
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
+
+    for kv in args.tune:
+        key, _, val = kv.partition("=")
+        if lib.msd_set_tuning(key.encode(), int(val)) != 0:
+            sys.exit("bench.py: " + lib.msd_last_error().decode())
 
     if args.calibrate_copy:
         src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()

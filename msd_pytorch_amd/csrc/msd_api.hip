@@ -14,9 +14,9 @@ namespace msd {
 const char *const kKnobNames[kKnobCount] = {
     "bwdx.vec2d", "bwdx.vec3d", "bwdx.unroll2d", "bwdx.unroll3d", "bwdx.min_blocks",
     "xcd_remap", "bwdk.vec2d", "bwdk.vec3d", "bwdk.blocks",
-    "fwd.vec2d", "fwd.vec3d", "fwd.split",
+    "fwd.vec2d", "fwd.vec3d", "fwd.split", "fwd.rows2d", "bwdk.rows",
 };
-int g_knobs[kKnobCount] = {-1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1};
+int g_knobs[kKnobCount] = {-1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1};
 int knob(Knob k, int dflt) { return g_knobs[k] < 0 ? dflt : g_knobs[k]; }
 }  // namespace msd
 
@@ -536,11 +536,6 @@ int msd_block_backward(int dtype, int ndim, int64_t batch, int64_t c_in, int dep
             MSD_TRY(msd_relu_mask_gradient(dtype, ndim, batch, w, spatial, out_i, stack_strides, gout_i,
                                            grads_strides, stream));
         masked = false;
-        if (i > 0 || need_input_grad)
-            MSD_TRY(backward_x("conv_backward_x", false, dtype, ndim, batch, first, w, spatial, (int)dilations[i],
-                               nullptr, nullptr, gout_i, grads_strides, weights[i], grads, grads_strides, stream,
-                               i > 0 ? (int)(first - widths[i - 1]) : (int)first, i > 0 ? stack : nullptr,
-                               stack_strides, &masked));
         void *gb = grad_bias ? (char *)grad_bias + b0 * a.elem : nullptr;
         if (grad_weights[i])
             MSD_TRY(backward_kb("conv_backward_kb", false, true, dtype, ndim, batch, first, w, spatial,
@@ -550,6 +545,11 @@ int msd_block_backward(int dtype, int ndim, int64_t batch, int64_t c_in, int dep
             MSD_TRY(backward_kb("conv_backward_bias", false, false, dtype, ndim, batch, 0, w, spatial, 1, nullptr,
                                 nullptr, gout_i, grads_strides, nullptr, nullptr, nullptr, gb, workspace,
                                 workspace_bytes, stream));
+        if (i > 0 || need_input_grad)
+            MSD_TRY(backward_x("conv_backward_x", false, dtype, ndim, batch, first, w, spatial, (int)dilations[i],
+                               nullptr, nullptr, gout_i, grads_strides, weights[i], grads, grads_strides, stream,
+                               i > 0 ? (int)(first - widths[i - 1]) : (int)first, i > 0 ? stack : nullptr,
+                               stack_strides, &masked));
         last = first;
         b1 = b0;
     }

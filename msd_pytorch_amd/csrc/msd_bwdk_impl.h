@@ -316,6 +316,282 @@ static __global__ __launch_bounds__(256) void reduce_columns(const float *__rest
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Row-team variant.  The gather of the A operands is the one backward_x uses (msd_rows.h): the
+// teams of a workgroup stage the source rows of their image rows in LDS once (coalesced V-wide
+// loads, the ReLU mask applied on the way in), and every lane takes the K taps of its own V
+// voxels from there.  From then on the waves are on their own, as above: LDS transpose into the
+// MFMA A layout, then the input channels in blocks of 16.  A workgroup walks `tiles_per_wg`
+// groups of rows and keeps its sums in registers until the end.
+
+template <int NDIM, int V> struct RowXTile {
+    static constexpr int kVox = kWave * V;
+    static constexpr int kStride = kVox + 4;
+    static constexpr int kRows = Taps<NDIM>::K > kChanBlock ? Taps<NDIM>::K : kChanBlock;
+    static constexpr int kFloats = kRows * kStride;
+};
+
+template <int NDIM, bool RELU, int V, int NCB>
+__global__ __launch_bounds__(kThreads, 2) void bwdk_rows(Geom g, RowTeams rt, int remap, int tiles_per_wg, int ngroups,
+                                                         int total_groups, View<const float> out,
+                                                         View<const float> gy, View<const float> x,
+                                                         float *__restrict__ part, int want_bias)
+{
+    extern __shared__ float lds[];
+    constexpr int K = Taps<NDIM>::K, NPQ = RowTaps<NDIM>::NPQ;
+    constexpr int TG = NDIM == 3 ? 2 : 1;         // groups of 16 tap rows
+    constexpr int NS = 4 * V;                     // 16-voxel MFMA groups per wave tile
+    constexpr int XSTRIDE = RowXTile<NDIM, V>::kStride;
+    const int tid = threadIdx.x;
+    const int nwaves = blockDim.x / kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave), wl = tid % kWave;
+    const int mk = wl / 16, mj = wl % 16;         // MFMA k (voxel) and i/j (tap or channel) of this lane
+    const int team = tid / rt.lpr, lane = tid % rt.lpr;
+    float *S = lds + (size_t)team * NPQ * V * rt.lpr;
+    float *XS = lds + (size_t)rt.rpw * NPQ * V * rt.lpr + (size_t)wave * RowXTile<NDIM, V>::kFloats;
+
+    const int co = blockIdx.z % g.Wd;
+    const int chunk = blockIdx.z / g.Wd;
+    const int c0 = chunk * NCB * kChanBlock;
+    const int ones_ch = want_bias ? g.C : -1;     // virtual channel of ones -> bias sum
+    const int c_end = min(g.C + (want_bias ? 1 : 0), c0 + NCB * kChanBlock);
+    const int ncb = (c_end - c0 + kChanBlock - 1) / kChanBlock;
+    // the staging code indexes output channels from 0: shift the views to this one
+    View<const float> outc = out, gyc = gy;
+    if (RELU) outc.p += (int64_t)co * out.sc;
+    gyc.p += (int64_t)co * gy.sc;
+
+    mfma4 D[NCB][TG];
+#pragma unroll
+    for (int cb = 0; cb < NCB; cb++)
+#pragma unroll
+        for (int tg = 0; tg < TG; tg++) D[cb][tg] = mfma4{0.f, 0.f, 0.f, 0.f};
+
+    const int lb = block_for_xcd(blockIdx.x, gridDim.x, remap);
+    const int x0 = lane * V;
+    const int xc = min(x0, g.W - V);
+
+    for (int ti = 0; ti < tiles_per_wg; ti++) {
+        const int grp = lb * tiles_per_wg + ti;
+        if (grp >= total_groups) break;           // uniform over the workgroup
+        int64_t xsc = x.sc;
+        asm volatile("" : "+s"(xsc));             // keeps the 16 channel offsets from being hoisted out of the loop
+        const int b = grp / ngroups;
+        const int row = (grp % ngroups) * rt.rpw + team;
+        const bool act = row < rt.nrows && x0 < g.W;
+        const int rr = min(row, rt.nrows - 1);
+        const int y = rr % g.H, z = rr / g.H;
+
+        // ---- input values of 16 channels for this lane's V voxels (B operand, before the transpose)
+        const float *xp0 = x.p + (int64_t)b * x.sb + (int64_t)z * x.sz + (int64_t)y * x.sy + xc;
+        float xv[kChanBlock][V];
+        auto load_block = [&](int cb) {
+            // branch-free: clamped channel index, all 16 loads in flight together
+#pragma unroll
+            for (int c = 0; c < kChanBlock; c++)
+                load_vec<V>(xp0 + (int64_t)min(c0 + cb * kChanBlock + c, g.C - 1) * xsc, xv[c]);
+        };
+        auto fix_block = [&](int cb) {
+#pragma unroll
+            for (int c = 0; c < kChanBlock; c++) {
+                const int ch = c0 + cb * kChanBlock + c;
+                const bool keep = act && ch < g.C;
+                const float fill = (act && ch == ones_ch) ? 1.f : 0.f;
+#pragma unroll
+                for (int i = 0; i < V; i++) xv[c][i] = keep ? xv[c][i] : fill;
+            }
+        };
+        load_block(0);   // issued ahead of the gather so the two latencies overlap
+
+        // ---- A operands, voxel layout: tv[t][i] = A[t](voxel x0 + i of the team's row)
+        {
+            float tv[K][V];
+            float own[1][NPQ][V];
+            stage_source_rows<NDIM, RELU, 1, V>(g, rt, outc, gyc, b, z, y, lane, act, S, own);
+#pragma unroll
+            for (int i = 0; i < V; i++) {
+                const SideTaps<V> side(min(x0 + i, g.W - 1), g.W, g.dil, rt.lpr);
+#pragma unroll
+                for (int pq = 0; pq < NPQ; pq++) {
+                    side.read(S + (size_t)pq * V * rt.lpr, tv[pq * 3 + 0][i], tv[pq * 3 + 2][i]);
+                    tv[pq * 3 + 1][i] = own[0][pq][i];
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < K; t++)
+#pragma unroll
+                for (int i = 0; i < V; i++) tv[t][i] = act ? tv[t][i] : 0.f;
+            __syncthreads();                      // the staged rows may be overwritten from here on
+            // through a wave-private LDS tile [tap][voxel] into the MFMA layout
+#pragma unroll
+            for (int t = 0; t < K; t++) store_vec<V>(XS + t * XSTRIDE + wl * V, tv[t]);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        // a[tg][s][e] = A[tap = tg*16 + mj](wave voxel 16 s + 4 mk + e)
+        float a[TG][NS][4];
+#pragma unroll
+        for (int tg = 0; tg < TG; tg++) {
+            const int tap = tg * 16 + mj;
+            const float *arow = XS + min(tap, K - 1) * XSTRIDE + 4 * mk;
+#pragma unroll
+            for (int s = 0; s < NS; s++) {
+                const f32x4 av = *reinterpret_cast<const f32x4 *>(arow + 16 * s);
+#pragma unroll
+                for (int e = 0; e < 4; e++) a[tg][s][e] = tap < K ? av[e] : 0.f;
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+        // ---- channel loop (runtime loop: unrolled, the addresses of all blocks would be live at once)
+#pragma unroll 1
+        for (int cb = 0; cb < ncb; cb++) {
+            fix_block(cb);
+#pragma unroll
+            for (int c = 0; c < kChanBlock; c++) store_vec<V>(XS + c * XSTRIDE + wl * V, xv[c]);
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            if (cb + 1 < ncb) load_block(cb + 1);   // in flight while the matrix cores work on this block
+            mfma4 acc[TG][2];                     // two independent accumulation chains per tap group
+#pragma unroll
+            for (int tg = 0; tg < TG; tg++) acc[tg][0] = acc[tg][1] = mfma4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < NS; s++) {
+                const f32x4 bv = *reinterpret_cast<const f32x4 *>(XS + mj * XSTRIDE + 16 * s + 4 * mk);
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+#pragma unroll
+                    for (int tg = 0; tg < TG; tg++)
+                        acc[tg][e & 1] =
+                            __builtin_amdgcn_mfma_f32_16x16x4f32(a[tg][s][e], bv[e], acc[tg][e & 1], 0, 0, 0);
+            }
+#pragma unroll
+            for (int q = 0; q < NCB; q++)
+                if (q == cb) {
+#pragma unroll
+                    for (int tg = 0; tg < TG; tg++) D[q][tg] += acc[tg][0] + acc[tg][1];
+                }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        }
+    }
+
+    // D[cb][tg][v] = sum for tap tg*16 + 4*mk + v, channel c0 + cb*16 + mj.  Add the waves in LDS.
+    __syncthreads();
+    constexpr int PER_WAVE = NCB * TG * 4 * kWave;
+    float *red = lds;
+#pragma unroll
+    for (int cb = 0; cb < NCB; cb++)
+#pragma unroll
+        for (int tg = 0; tg < TG; tg++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) red[wave * PER_WAVE + ((cb * TG + tg) * 4 + v) * kWave + wl] = D[cb][tg][v];
+    __syncthreads();
+    float *pcol = part + blockIdx.x;
+    for (int idx = tid; idx < PER_WAVE; idx += blockDim.x) {
+        const int l = idx % kWave, v = (idx / kWave) % 4, tg = (idx / (4 * kWave)) % TG, cb = idx / (4 * kWave * TG);
+        const int tap = tg * 16 + 4 * (l / 16) + v;
+        const int ch = c0 + cb * kChanBlock + l % 16;
+        if (tap >= K || ch >= c_end) continue;
+        float s = 0.f;
+        for (int w = 0; w < nwaves; w++) s += red[w * PER_WAVE + idx];
+        if (ch < g.C)
+            pcol[(((int64_t)co * g.C + ch) * K + tap) * kMaxPartialRows] = s;
+        else if (tap == K / 2)
+            pcol[((int64_t)g.Wd * g.C * K + co) * kMaxPartialRows] = s;
+    }
+}
+
+template <int NDIM, int V, int NCB>
+size_t rows_lds_bytes(const RowTeams &rt)
+{
+    constexpr int TG = NDIM == 3 ? 2 : 1;
+    const size_t main_loop =
+        ((size_t)rt.rpw * RowTaps<NDIM>::NPQ * V * rt.lpr + (size_t)kWaves * RowXTile<NDIM, V>::kFloats) * 4;
+    const size_t epilogue = (size_t)kWaves * NCB * TG * 4 * kWave * 4;
+    return std::max(main_loop, epilogue);
+}
+
+// Row-team kernel usable: rows fit a 256-lane workgroup, V-wide accesses aligned.
+template <int NDIM>
+bool rows_fit(const Geom &g, bool relu, int V, const View<const float> &out, const View<const float> &gy,
+              const View<const float> &x)
+{
+    RowTeams rt;
+    if (!make_row_teams(g, V, &rt) || rt.lpr * rt.rpw > kThreads) return false;
+    if (!rows_aligned(x, g.W, V) || !rows_aligned(gy, g.W, V) || (relu && !rows_aligned(out, g.W, V))) return false;
+    return g.W >= V;
+}
+
+template <int NDIM, bool RELU, int V, int NCB>
+hipError_t launch_rows(const Geom &g, const View<const float> &out, const View<const float> &gy,
+                       const View<const float> &x, float *gk, float *gb, float *ws, hipStream_t s)
+{
+    constexpr int K = Taps<NDIM>::K;
+    RowTeams rt;
+    make_row_teams(g, V, &rt);
+    float *part = ws + backward_k_mask_floats(g);
+    const int ngroups = (rt.nrows + rt.rpw - 1) / rt.rpw;
+    const int64_t total = (int64_t)ngroups * g.B;
+    const int remap = knob(kKnobXcdRemap, 1);
+    const int64_t max_wgs = std::min<int64_t>(std::max(8, knob(kKnobBwdkBlocks, kMaxPartialRows)), kMaxPartialRows);
+    const int tiles_per_wg = (int)((total + max_wgs - 1) / max_wgs);
+    const int64_t wgs = (total + tiles_per_wg - 1) / tiles_per_wg;
+    const int rows = remap ? xcd_grid((int)wgs) : (int)wgs;   // padding workgroups write zero rows
+    if (rows > kMaxPartialRows || total > INT32_MAX) return hipErrorInvalidConfiguration;
+    const int want_bias = gb != nullptr;
+    const int chunks = (g.C + want_bias + NCB * kChanBlock - 1) / (NCB * kChanBlock);
+    const size_t lds = rows_lds_bytes<NDIM, V, NCB>(rt);
+    hipLaunchKernelGGL((bwdk_rows<NDIM, RELU, V, NCB>), dim3(rows, 1, chunks * g.Wd), dim3(rt.lpr * rt.rpw), lds, s, g,
+                       rt, remap, tiles_per_wg, ngroups, (int)total, out, gy, x, part, want_bias);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    const int64_t nk = (int64_t)g.Wd * g.C * K;
+    const int64_t ncols = nk + (want_bias ? g.Wd : 0);
+    hipLaunchKernelGGL(reduce_columns, dim3((ncols + 3) / 4), dim3(256), 0, s, part, rows, nk, ncols, gk, gb);
+    return hipGetLastError();
+}
+
+template <int NDIM, bool RELU, int V>
+hipError_t rows_pick_ncb(const Geom &g, const View<const float> &out, const View<const float> &gy,
+                         const View<const float> &x, float *gk, float *gb, float *ws, hipStream_t s)
+{
+    const int need = (g.C + (gb != nullptr) + kChanBlock - 1) / kChanBlock;
+    if (need <= 1) return launch_rows<NDIM, RELU, V, 1>(g, out, gy, x, gk, gb, ws, s);
+    if (need <= 2) return launch_rows<NDIM, RELU, V, 2>(g, out, gy, x, gk, gb, ws, s);
+    if (need <= 4) return launch_rows<NDIM, RELU, V, 4>(g, out, gy, x, gk, gb, ws, s);
+    return launch_rows<NDIM, RELU, V, 8>(g, out, gy, x, gk, gb, ws, s);
+}
+
+// Voxels per lane of the row-team kernel: the widest aligned one up to vmax, 0 if none fits.
+template <int NDIM>
+int rows_choose_vec(const Geom &g, bool relu, int vmax, const View<const float> &out, const View<const float> &gy,
+                    const View<const float> &x)
+{
+    for (int v = NDIM == 3 ? 2 : 4; v >= 1; v /= 2) {
+        if (v > vmax) continue;
+        if (rows_fit<NDIM>(g, relu, v, out, gy, x)) return v;
+    }
+    return 0;
+}
+
+template <int NDIM, bool RELU>
+hipError_t rows_run(const Geom &g, int v, const View<const float> &out, const View<const float> &gy,
+                    const View<const float> &x, float *gk, float *gb, float *ws, hipStream_t s)
+{
+    if constexpr (NDIM == 2) {
+        if (v == 4) return rows_pick_ncb<2, RELU, 4>(g, out, gy, x, gk, gb, ws, s);
+    }
+    if (v == 2) return rows_pick_ncb<NDIM, RELU, 2>(g, out, gy, x, gk, gb, ws, s);
+    if (v == 1) return rows_pick_ncb<NDIM, RELU, 1>(g, out, gy, x, gk, gb, ws, s);
+    return hipErrorInvalidConfiguration;
+}
+
 template <int NDIM, int V, int NCB>
 size_t lds_bytes()
 {
@@ -390,7 +666,7 @@ bool supported_nd(const Geom &g, bool relu, const View<const float> &out, const 
                   const View<const float> &x)
 {
     if (x.sx != 1 || gy.sx != 1 || (relu && out.sx != 1)) return false;
-    return choose_vec(g, 4, x) != 0;
+    return rows_choose_vec<NDIM>(g, relu, 4, out, gy, x) != 0 || choose_vec(g, 4, x) != 0;
 }
 
 template <int NDIM>
@@ -398,6 +674,13 @@ hipError_t run_nd(const Geom &g, bool relu, const View<const float> &out, const 
                   const View<const float> &x, float *gk, float *gb, float *ws, hipStream_t s)
 {
     const int vmax = knob(NDIM == 3 ? kKnobBwdkVec3d : kKnobBwdkVec2d, NDIM == 3 ? 2 : 4);
+    if (knob(kKnobBwdkRows, 1)) {
+        int rv = rows_choose_vec<NDIM>(g, relu, vmax, out, gy, x);
+        if (rv == 0) rv = rows_choose_vec<NDIM>(g, relu, 4, out, gy, x);
+        if (rv != 0)
+            return relu ? rows_run<NDIM, true>(g, rv, out, gy, x, gk, gb, ws, s)
+                        : rows_run<NDIM, false>(g, rv, out, gy, x, gk, gb, ws, s);
+    }
     int v = choose_vec(g, vmax, x);
     if (v == 0) v = choose_vec(g, 4, x);
     if (v == 4) return pick_ncb<NDIM, 4>(g, relu, out, gy, x, gk, gb, ws, s);

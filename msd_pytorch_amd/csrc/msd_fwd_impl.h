@@ -73,6 +73,10 @@ __global__ __launch_bounds__(1024) void fwd_lattice(Geom g, Lattice lt, int rema
     for (int m = 0; m < LY; m++)
         offy[m] = (int64_t)min(reflect_idx(min(y0 + (m - 1) * g.dil, 2 * g.H - 1), g.H), g.H - 1) * x.sy;
 
+    // valid output rows of this lattice (the rest lie past the image edge)
+    const int nyv = min(RY, (g.H - y0 + g.dil - 1) / g.dil);
+    const int nzv = NDIM == 3 ? min(RZ, (g.D - z0 + g.dil - 1) / g.dil) : 1;
+
     float acc[WOUT][RZ][RY][3][V];
 #pragma unroll
     for (int co = 0; co < WOUT; co++)
@@ -93,31 +97,35 @@ __global__ __launch_bounds__(1024) void fwd_lattice(Geom g, Lattice lt, int rema
         for (int co = 0; co < WOUT; co++)
 #pragma unroll
             for (int t = 0; t < K; t++) w[co][t] = k[((int64_t)co * g.C + ci) * K + t];
+        // all row loads of this channel are issued before the first multiply-add
+        float xv[LZ][LY][V];
 #pragma unroll
         for (int mz = 0; mz < LZ; mz++)
 #pragma unroll
-            for (int my = 0; my < LY; my++) {
-                float xv[V];
-                load_vec<V>(xc + offz[mz] + offy[my], xv);
+            for (int my = 0; my < LY; my++) load_vec<V>(xc + offz[mz] + offy[my], xv[mz][my]);
+        if constexpr (WOUT == 1) __builtin_amdgcn_sched_barrier(0);
+        // output rows past the image edge (partial lattices) are skipped, uniformly per workgroup
 #pragma unroll
-                for (int p = 0; p < NZ; p++) {
-                    const int jz = NDIM == 3 ? mz - p : 0;       // input level m = j + p  (p, q counted from 0)
-                    if (jz < 0 || jz >= RZ) continue;
+        for (int jz = 0; jz < RZ; jz++) {
+            if (jz >= nzv) break;
 #pragma unroll
-                    for (int q = 0; q < 3; q++) {
-                        const int jy = my - q;
-                        if (jy < 0 || jy >= RY) continue;
+            for (int jy = 0; jy < RY; jy++) {
+                if (jy >= nyv) break;
+#pragma unroll
+                for (int p = 0; p < NZ; p++)
+#pragma unroll
+                    for (int q = 0; q < 3; q++)
 #pragma unroll
                         for (int co = 0; co < WOUT; co++)
 #pragma unroll
                             for (int r = 0; r < 3; r++) {
                                 const float wv = w[co][(p * 3 + q) * 3 + r];
 #pragma unroll
-                                for (int i = 0; i < V; i++) acc[co][jz][jy][r][i] += xv[i] * wv;
+                                for (int i = 0; i < V; i++)
+                                    acc[co][jz][jy][r][i] += xv[NDIM == 3 ? jz + p : 0][jy + q][i] * wv;
                             }
-                    }
-                }
             }
+        }
     }
 
     // Finish the rows one at a time.  LDS holds T_r of the current row for every
@@ -239,6 +247,21 @@ hipError_t pick(const Geom &g, const View<const float> &x, const float *k, const
         if (v == 2) return launch<3, RELU, WOUT, 2, 2, 4>(g, x, k, bias, out, s);
         if (v == 1) return launch<3, RELU, WOUT, 1, 2, 4>(g, x, k, bias, out, s);
     } else {
+        if (v == 4 && WOUT == 1) {
+            // Rows per tile: all tiles cost the same, so the time is (rounds of tiles over
+            // the 256 CUs) x (rows per tile); with few tiles a longer chain that avoids a
+            // nearly empty last round wins.
+            int best = 4;
+            long best_cost = 0;
+            for (int ry = 4; ry <= 6; ry++) {
+                const long tiles = (long)g.dil * (((g.H + g.dil - 1) / g.dil + ry - 1) / ry) * g.B;
+                const long cost = (tiles + 255) / 256 * ry;
+                if (ry == 4 || cost < best_cost) { best = ry; best_cost = cost; }
+            }
+            best = knob(kKnobFwdRows2d, best);
+            if (best == 5) return launch<2, RELU, 1, 4, 1, 5>(g, x, k, bias, out, s);
+            if (best == 6) return launch<2, RELU, 1, 4, 1, 6>(g, x, k, bias, out, s);
+        }
         if (v == 4) return launch<2, RELU, WOUT, 4, 1, 4>(g, x, k, bias, out, s);
         if (v == 2) return launch<2, RELU, WOUT, 2, 1, 4>(g, x, k, bias, out, s);
         if (v == 1) return launch<2, RELU, WOUT, 1, 1, 4>(g, x, k, bias, out, s);

@@ -7,7 +7,7 @@ namespace msd {
 
 // Upper bound on the number of partial-sum rows of the weight/bias gradient
 // reduction (one row per workgroup of the first pass).
-constexpr int kMaxPartialRows = 512;
+constexpr int kMaxPartialRows = 1024;
 
 // Elements at the start of the workspace that hold the masked output gradient
 // of the matrix-core backward_k (a multiple of 64 so the partial sums behind it
@@ -38,7 +38,7 @@ hipError_t generic_backward_kb(const Geom &g, bool relu, View<const T> out, View
 enum Knob {
     kKnobBwdxVec2d, kKnobBwdxVec3d, kKnobBwdxUnroll2d, kKnobBwdxUnroll3d, kKnobBwdxMinBlocks,
     kKnobXcdRemap, kKnobBwdkVec2d, kKnobBwdkVec3d, kKnobBwdkBlocks,
-    kKnobFwdVec2d, kKnobFwdVec3d, kKnobFwdSplit,
+    kKnobFwdVec2d, kKnobFwdVec3d, kKnobFwdSplit, kKnobFwdRows2d, kKnobBwdkRows,
     kKnobCount
 };
 int knob(Knob k, int dflt);
