@@ -77,21 +77,28 @@ def make_model(name, torch):
     return model
 
 
-def algorithmic_bytes(name):
-    """Per-step algorithmic bytes of each kernel class, fp32:
-    forward (C + w) N 4, backward_x (2C + 2w) N 4, backward_k+bias (C + 2w) N 4,
-    each plus the w*C*K weights."""
+def algorithmic_bytes(name, fused):
+    """Per-step algorithmic bytes of each kernel class, fp32, per layer with C input and
+    w output channels over N voxels:
+    forward (C + w) N 4, backward_x (2C + 2w) N 4, backward_k+bias (C + 2w) N 4, the fused
+    backward_x + backward_k+bias pass (3C + 2w) N 4, each plus the w*C*K weights; the
+    separate ReLU-mask pass of the top layer 3 w N 4 (counted with backward_x).
+    `fused` says which way the library ran the layers above the first (it reports a
+    non-zero call count for the fused class); layer 0 needs no input gradient."""
     kind, ndim, c_in, c_out, depth, width, batch, spatial, adam = WORKLOADS[name]
     n = batch
     for s in spatial:
         n *= s
     K = 3 ** ndim
-    out = {"forward": 0, "backward_x": 0, "backward_kb": 0}
+    out = {"forward": 0, "backward_x": 3 * width * n * 4, "backward_kb": 0, "backward_xkb": 0}
     for i in range(depth):
         C = c_in + width * i
         wts = width * C * K * 4
         out["forward"] += (C + width) * n * 4 + wts
-        if i > 0:   # layer 0's input gradient is not needed (the network input is data)
+        if i > 0 and fused:
+            out["backward_xkb"] += (3 * C + 2 * width) * n * 4 + 2 * wts
+            continue
+        if i > 0:
             out["backward_x"] += (2 * C + 2 * width) * n * 4 + wts
         out["backward_kb"] += (C + 2 * width) * n * 4 + wts
     return out, n
@@ -105,13 +112,13 @@ def kernel_times(lib, torch, run_steps):
     lib.msd_profile_enable(1)
     run_steps()
     torch.cuda.synchronize()
-    ms = (ctypes.c_double * 3)()
-    calls = (ctypes.c_int64 * 3)()
+    ms = (ctypes.c_double * 4)()
+    calls = (ctypes.c_int64 * 4)()
     rc = lib.msd_profile_read(ms, calls)
     lib.msd_profile_enable(0)
     if rc != 0:
         raise RuntimeError(lib.msd_last_error().decode())
-    names = ("forward", "backward_x", "backward_kb")
+    names = ("forward", "backward_x", "backward_kb", "backward_xkb")
     return {n: (ms[i], calls[i]) for i, n in enumerate(names)}
 
 
@@ -211,7 +218,7 @@ def main():
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed / args.steps * 1e3
 
-    bytes_per_step, nvox = algorithmic_bytes(name)
+    _, nvox = algorithmic_bytes(name, False)
     result = {
         "metric": "MSD train-step Mvoxel/s",
         "value": round(nvox / (ms_per_step * 1e-3) / 1e6, 3),
@@ -226,6 +233,7 @@ def main():
 
     if not args.no_kernel_timing:
         totals = kernel_times(lib, torch, lambda: [step() for _ in range(args.steps)])
+        bytes_per_step, _ = algorithmic_bytes(name, totals["backward_xkb"][1] > 0)
         kernels = {}
         for cls, (ms, launches) in totals.items():
             if launches == 0:

@@ -220,10 +220,12 @@ int msd_block_backward(int dtype, int ndim, int64_t batch, int64_t c_in, int dep
  * Kernel timing for benchmarks.  While enabled, every operator call (also inside
  * the block calls) is bracketed by HIP events recorded on its launch stream.
  * msd_profile_read waits for the recorded events and returns, per class
- * {0 forward, 1 backward_x incl. the mask, 2 backward_k/bias}, the summed elapsed
- * milliseconds and the number of calls since msd_profile_enable(1).  Not thread-safe;
- * no counterpart in the reference.
+ * {0 forward, 1 backward_x incl. the mask, 2 backward_k/bias, 3 fused backward_x +
+ * backward_k/bias of the block backward pass}, the summed elapsed milliseconds and the
+ * number of calls since msd_profile_enable(1); ms and calls hold
+ * MSD_PROFILE_CLASSES entries.  Not thread-safe; no counterpart in the reference.
  */
+#define MSD_PROFILE_CLASSES 4
 int msd_profile_enable(int on);
 int msd_profile_read(double *ms, int64_t *calls);
 

@@ -14,9 +14,9 @@ namespace msd {
 const char *const kKnobNames[kKnobCount] = {
     "bwdx.vec2d", "bwdx.vec3d", "bwdx.unroll2d", "bwdx.unroll3d", "bwdx.min_blocks",
     "xcd_remap", "bwdk.vec2d", "bwdk.vec3d", "bwdk.blocks",
-    "fwd.vec2d", "fwd.vec3d", "fwd.split", "fwd.rows2d", "bwdk.rows",
+    "fwd.vec2d", "fwd.vec3d", "fwd.split", "fwd.rows2d", "bwdk.rows", "block.fuse",
 };
-int g_knobs[kKnobCount] = {-1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1};
+int g_knobs[kKnobCount] = {-1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1};
 int knob(Knob k, int dflt) { return g_knobs[k] < 0 ? dflt : g_knobs[k]; }
 }  // namespace msd
 
@@ -32,11 +32,13 @@ template <> struct is_f32<float> { static constexpr bool value = true; };
 
 // Optional per-class kernel timing with HIP events recorded on the launch stream
 // (msd_profile_* in the C ABI).  Classes: 0 forward, 1 backward_x (+ mask), 2 backward_k/bias.
+constexpr int kProfileClasses = 4;   // forward, backward_x, backward_k(+bias), fused backward_x+k
+
 struct Profile {
     bool on = false;
     std::vector<hipEvent_t> pool;                           // reused across calls
     size_t used = 0;
-    std::vector<std::pair<size_t, size_t>> spans[3];        // (start, stop) indices into pool
+    std::vector<std::pair<size_t, size_t>> spans[kProfileClasses];        // (start, stop) indices into pool
     hipEvent_t take()
     {
         if (used == pool.size()) {
@@ -471,6 +473,46 @@ int check_block(const char *fn, int dtype, int ndim, int64_t batch, int64_t c_in
     return MSD_OK;
 }
 
+
+// One layer of the block backward pass with the fused kernel: grad_input channels
+// [0, first) += backward_x, grad_weights/grad_bias += backward_k/bias, the ReLU mask of the
+// layer below applied to its channels on the way out.  *done is false (and nothing was
+// launched) when the fused kernel does not cover the case.
+int block_layer_fused(const char *fn, const BlockArgs &a, int i, int64_t first, const void *stack,
+                      const int64_t *stack_strides, void *grads, const int64_t *grads_strides, const void *gout_i,
+                      const void *weights_i, void *gk, void *gb, void *ws, int64_t ws_bytes, hipStream_t s,
+                      bool *masked, bool *done)
+{
+    *done = false;
+    if (a.dtype != MSD_F32 || g_kernel_path != 0 || !gk || !msd::knob(msd::kKnobBlockFuse, 1)) return MSD_OK;
+    msd::Geom g;
+    MSD_TRY(make_geom(fn, a.dtype, a.ndim, a.batch, first, a.widths[i], a.spatial, (int)a.dilations[i], true, &g));
+    msd::View<const float> gy, x;
+    msd::View<float> gx;
+    MSD_TRY(make_view(fn, "grad_output", a.ndim, gout_i, grads_strides, &gy));
+    MSD_TRY(make_view(fn, "input", a.ndim, stack, stack_strides, &x));
+    MSD_TRY(make_view(fn, "grad_input", a.ndim, grads, grads_strides, &gx));
+    if (!msd::fast_backward_xkb_supported(g, gy, x, gx)) return MSD_OK;
+    MSD_TRY(check_workspace(fn, g, sizeof(float), ws, ws_bytes));
+    msd::PostMask pm{g.C, {nullptr, 0, 0, 0, 0, 0}};
+    *masked = false;
+    if (i > 0) {
+        // the activations are read through grad_input's addressing: same strides and alignment
+        const bool same_layout = x.sb == gx.sb && x.sc == gx.sc && x.sz == gx.sz && x.sy == gx.sy &&
+                                 reinterpret_cast<uintptr_t>(x.p) % 16 == reinterpret_cast<uintptr_t>(gx.p) % 16;
+        if (same_layout) {
+            pm = msd::PostMask{(int)(first - a.widths[i - 1]), x};
+            *masked = true;
+        }
+    }
+    ProfileScope scope(3, s);
+    const hipError_t e = msd::fast_backward_xkb(g, gy, x, (const float *)weights_i, gx, pm, (float *)gk, (float *)gb,
+                                                (float *)ws, s);
+    if (e != hipSuccess) return hip_fail(fn, e);
+    *done = true;
+    return MSD_OK;
+}
+
 }  // namespace
 
 int64_t msd_block_workspace_bytes(int dtype, int ndim, int64_t batch, int64_t c_in, int depth, const int64_t *widths,
@@ -537,6 +579,18 @@ int msd_block_backward(int dtype, int ndim, int64_t batch, int64_t c_in, int dep
                                            grads_strides, stream));
         masked = false;
         void *gb = grad_bias ? (char *)grad_bias + b0 * a.elem : nullptr;
+        if (i > 0 || need_input_grad) {
+            // one pass for the input, weight and bias gradients where the fused kernel applies
+            bool done = false;
+            MSD_TRY(block_layer_fused(fn, a, i, first, stack, stack_strides, grads, grads_strides, gout_i, weights[i],
+                                      grad_weights[i], gb, workspace, workspace_bytes, (hipStream_t)stream, &masked,
+                                      &done));
+            if (done) {
+                last = first;
+                b1 = b0;
+                continue;
+            }
+        }
         if (grad_weights[i])
             MSD_TRY(backward_kb("conv_backward_kb", false, true, dtype, ndim, batch, first, w, spatial,
                                 (int)dilations[i], nullptr, nullptr, gout_i, grads_strides, stack, stack_strides,
@@ -567,7 +621,7 @@ int msd_profile_enable(int on)
 int msd_profile_read(double *ms, int64_t *calls)
 {
     if (!ms || !calls) return fail(MSD_ERR_INVALID, "msd_profile_read: NULL argument");
-    for (int c = 0; c < 3; c++) {
+    for (int c = 0; c < kProfileClasses; c++) {
         double total = 0;
         for (const auto &sp : g_profile.spans[c]) {
             hipError_t e = hipEventSynchronize(g_profile.pool[sp.second]);

@@ -1,0 +1,448 @@
+// backward_x and backward_k (+ bias) of one layer in a single pass over the input
+// channels, fp32, unit x-stride, one output channel, output gradient already masked:
+//     grad_input[ci][u] += sum_t k[ci][t] * A[t](u)
+//     grad_kernel[ci][t] += sum_u x[ci][u] * A[t](u),     grad_bias += sum_u A[centre](u)
+// Both need the same adjoint-form gather A[t](u) of the output gradient (msd_adjoint.h,
+// msd_rows.h); done once per tile of rows, it then serves a stream over the input
+// channels that reads x[ci], reads and writes grad_input[ci], and touches nothing else.
+//
+// Work split.  Row teams as in msd_rows.h: a team of lpr lanes (a multiple of 64 here)
+// owns an image row, a lane V consecutive voxels of it, so a WAVE owns 64*V consecutive
+// voxels.  After the gather every lane holds A[t] of its own voxels in registers
+// ("voxel layout"): that is what the grad_input update needs, K*V fused multiply-adds
+// per channel with wave-uniform weights.  The weight gradient is a contraction over
+// voxels and goes to the matrix cores, v_mfma_f32_16x16x4_f32 with taps as rows,
+// 16 input channels as columns and 4 voxels per instruction:
+//   A operand  the wave writes its A[t][voxel] tile to a private LDS tile once per row
+//              tile and reads 4-voxel groups of row `tap` back per instruction;
+//   B operand  lane (channel j, voxel group k) loads x[c0 + j][16 s + 4 k ...+3] straight
+//              from memory as one 16-byte access: the layout change costs nothing.
+// The channel loop is software-pipelined in stages of 32 or 64 of the wave's voxels for
+// 16 channels of x plus 8 or 4 channels of grad_input: the loads of the next stage are
+// issued before the arithmetic of the current one, into the other of two register sets.
+// Partial sums of the weight gradient stay in registers over all row tiles of a
+// workgroup, are added over its waves in LDS and leave as one column-major row per
+// workgroup; bwdk::reduce_columns adds the rows in a fixed order.
+//
+// Registers.  Kernel arguments live in scalar registers for the whole kernel, so they
+// are kept small: 32-bit strides (checked on the host), no view that is not read.
+// grad_input is addressed as a wave-uniform channel base plus a 32-bit lane offset, which
+// costs no vector registers or vector arithmetic per channel.
+// Algorithmic traffic: (3C + 2w) * N * 4 bytes.
+#pragma once
+#include "msd_bwdk_impl.h"
+
+#include <type_traits>
+
+namespace msd {
+namespace bwdxk {
+
+using bwdk::kChanBlock;
+using bwdk::kThreads;
+using bwdk::kWaves;
+using bwdk::mfma4;
+
+// Wave-private LDS tile [tap][voxel]; one more row of zeros feeds the MFMA rows past K.
+template <int NDIM, int V> struct ATile {
+    static constexpr int kStride = kWave * V + 4;     // floats per row (bank spread for the b128 reads)
+    static constexpr int kRows = Taps<NDIM>::K + 1;
+    static constexpr int kFloats = kRows * kStride;
+};
+
+// Element strides {batch, channel, z, y} of a tensor; the x stride is 1.
+struct Plane {
+    int sb, sc, sz, sy;
+};
+
+struct Args {
+    Geom g;
+    RowTeams rt;
+    int remap, tiles_per_wg, ngroups, total_groups;
+    Plane gy;            // masked output gradient, one channel (sc unused)
+    Plane x;             // input channels
+    Plane gx;            // grad_input channels (written through a cast)
+    int mask_from;       // activations (viewed like grad_input) mask the channels >= mask_from
+    int want_bias;
+};
+
+template <int NDIM, int V, int NCB>
+__global__ __launch_bounds__(kThreads, 2) void bwd_rows_fused(const Args a, const float *__restrict__ gyp,
+                                                              const float *__restrict__ xp, float *__restrict__ gxp,
+                                                              const float *__restrict__ actp,
+                                                              const float *__restrict__ kw, float *__restrict__ part)
+{
+    // the pointers are separate arguments so that they can carry __restrict__: the weights
+    // are then known not to change under the stores to grad_input and stay scalar loads
+    extern __shared__ float lds[];
+    constexpr int K = Taps<NDIM>::K, NPQ = RowTaps<NDIM>::NPQ;
+    constexpr int TG = NDIM == 3 ? 2 : 1;         // groups of 16 tap rows
+    constexpr int NSS = V == 1 ? 2 : 4;           // 16-voxel MFMA groups per pipeline stage
+    constexpr int H = 4 * V / NSS;                // stages per block of 16 channels (even)
+    constexpr int NCS = kChanBlock / H;           // grad_input channels per stage
+    constexpr int ASTRIDE = ATile<NDIM, V>::kStride;
+    const Geom &g = a.g;
+    const RowTeams &rt = a.rt;
+    const int tid = threadIdx.x;
+    const int nwaves = blockDim.x / kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave), wl = tid % kWave;
+    const int mk = wl / 16, mj = wl % 16;         // MFMA k (voxel group) and i/j (tap or channel) of this lane
+    const int team = tid / rt.lpr, lane = tid % rt.lpr;
+    float *S = lds + (size_t)team * NPQ * V * rt.lpr;
+    float *AT = lds + (size_t)rt.rpw * NPQ * V * rt.lpr + (size_t)wave * ATile<NDIM, V>::kFloats;
+    for (int i = wl; i < ASTRIDE; i += kWave) AT[K * ASTRIDE + i] = 0.f;
+
+    const int c0 = blockIdx.z * NCB * kChanBlock;
+    const int ones_ch = a.want_bias ? g.C : -1;   // virtual channel of ones -> bias sum
+    const int c_end = min(g.C + (a.want_bias ? 1 : 0), c0 + NCB * kChanBlock);
+    const int cx_end = min(c_end, g.C);           // real channels of this chunk end here
+    const int ncb = (c_end - c0 + kChanBlock - 1) / kChanBlock;
+
+    mfma4 D[NCB][TG];
+#pragma unroll
+    for (int cb = 0; cb < NCB; cb++)
+#pragma unroll
+        for (int tg = 0; tg < TG; tg++) D[cb][tg] = mfma4{0.f, 0.f, 0.f, 0.f};
+
+    const int lb = block_for_xcd(blockIdx.x, gridDim.x, a.remap);
+    const int x0 = lane * V;
+    const int xc = min(x0, g.W - V);
+    const int kx = (lane - wl) * V + 4 * mk;      // first voxel of this lane's MFMA groups, + 16 s
+    int arow[TG];                                 // this lane's row of the A tile (the zero row past K taps)
+#pragma unroll
+    for (int tg = 0; tg < TG; tg++) arow[tg] = min(tg * 16 + mj, K) * ASTRIDE + 4 * mk;
+
+    for (int ti = 0; ti < a.tiles_per_wg; ti++) {
+        const int grp = lb * a.tiles_per_wg + ti;
+        if (grp >= a.total_groups) break;         // uniform over the workgroup
+        int xsc = a.x.sc, gsc = a.gx.sc;
+        asm volatile("" : "+s"(xsc), "+s"(gsc));  // keeps per-channel addresses from being hoisted out of the loop
+        const int b = grp / a.ngroups;
+        const int row = (grp % a.ngroups) * rt.rpw + team;
+        const bool rowok = row < rt.nrows;
+        const bool act = rowok && x0 < g.W;
+        const int rr = min(row, rt.nrows - 1);
+        const int y = rr % g.H, z = rr / g.H;
+        // x: per-lane channel, so a full address per lane
+        const float *xk = xp + (int64_t)b * a.x.sb + (int64_t)z * a.x.sz + (int64_t)y * a.x.sy;
+        // grad_input and activations: uniform base of (batch, channel) + byte offset of the lane's voxels
+        char *gbase = reinterpret_cast<char *>(gxp + (int64_t)b * a.gx.sb);
+        const char *abase = reinterpret_cast<const char *>(actp + (int64_t)b * a.gx.sb);
+        const uint32_t goff = 4u * (uint32_t)(z * a.gx.sz + y * a.gx.sy + xc);
+
+        // ---- one pipeline stage of loads: NSS 16-voxel groups of 16 channels of x in the MFMA B
+        // layout, and NCS channels of grad_input in the voxel layout.  Clamped, always valid
+        // addresses; what does not count is replaced after the load.
+        float ka[NSS][4], kb[NSS][4];             // stages alternate between the a and b buffers
+        float ga[NCS][V], gb[NCS][V];
+        auto load_stage = [&](int cb, int h, float (&kk)[NSS][4], float (&gg)[NCS][V]) {
+            const float *p = xk + (int64_t)min(c0 + cb * kChanBlock + mj, g.C - 1) * xsc;
+#pragma unroll
+            for (int j = 0; j < NSS; j++) {
+                const f32x4 v = *reinterpret_cast<const f32x4 *>(p + min(kx + 16 * (h * NSS + j), g.W - 4));
+#pragma unroll
+                for (int e = 0; e < 4; e++) kk[j][e] = v[e];
+            }
+#pragma unroll
+            for (int j = 0; j < NCS; j++) {
+                const int ci = max(min(c0 + cb * kChanBlock + h * NCS + j, cx_end - 1), 0);
+                load_vec<V>(reinterpret_cast<const float *>(gbase + (int64_t)ci * gsc * 4 + goff), gg[j]);
+            }
+        };
+        load_stage(0, 0, ka, ga);   // issued ahead of the gather so the two latencies overlap
+
+        // ---- A operands, voxel layout: tv[t][i] = A[t](voxel x0 + i of the team's row)
+        float tv[K][V];
+        {
+            const View<const float> none{nullptr, 0, 0, 0, 0, 0};
+            const View<const float> gyv{gyp, a.gy.sb, 0, a.gy.sz, a.gy.sy, 1};
+            float own[1][NPQ][V];
+            stage_source_rows<NDIM, false, 1, V>(g, rt, none, gyv, b, z, y, lane, act, S, own);
+            // per voxel: all LDS reads first, so that their latencies overlap, then the sums
+#pragma unroll
+            for (int i = 0; i < V; i++) {
+                const SideTaps<V> side(min(x0 + i, g.W - 1), g.W, g.dil, rt.lpr);
+                float ra[NPQ][4];
+#pragma unroll
+                for (int pq = 0; pq < NPQ; pq++) {
+                    const float *srow = S + (size_t)pq * V * rt.lpr;
+                    ra[pq][0] = srow[side.i0a];
+                    ra[pq][1] = srow[side.i0b];
+                    ra[pq][2] = srow[side.i2a];
+                    ra[pq][3] = srow[side.i2b];
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int pq = 0; pq < NPQ; pq++) {
+                    tv[pq * 3 + 0][i] = (side.m0a ? ra[pq][0] : 0.f) + (side.m0b ? ra[pq][1] : 0.f);
+                    tv[pq * 3 + 1][i] = own[0][pq][i];
+                    tv[pq * 3 + 2][i] = (side.m2a ? ra[pq][2] : 0.f) + (side.m2b ? ra[pq][3] : 0.f);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            __syncthreads();                      // the staged rows may be overwritten from here on
+            // the wave's [tap][voxel] tile; lanes past the row hold finite values that meet zeros of x
+#pragma unroll
+            for (int t = 0; t < K; t++) store_vec<V>(AT + t * ASTRIDE + wl * V, tv[t]);
+        }
+        // the tile is private to the wave and LDS executes a wave's accesses in order: only
+        // the compiler has to be kept from reordering them
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+        mfma4 acc[TG][2];                         // two independent accumulation chains per tap group
+        // weight gradient of one stage: 4 * NSS * TG matrix instructions
+        auto stage_k = [&](int cb, int h, float (&kk)[NSS][4]) {
+            const int chl = c0 + cb * kChanBlock + mj;
+            const bool chok = chl < g.C, one = chl == ones_ch;
+#pragma unroll
+            for (int j = 0; j < NSS; j++) {
+                const int s = h * NSS + j;
+                const bool vok = rowok && kx + 16 * s < g.W;
+                const bool keep = vok && chok;
+                const float fill = (vok && one) ? 1.f : 0.f;
+                f32x4 av[TG];
+#pragma unroll
+                for (int tg = 0; tg < TG; tg++) av[tg] = *reinterpret_cast<const f32x4 *>(AT + arow[tg] + 16 * s);
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const float bv = keep ? kk[j][e] : fill;
+#pragma unroll
+                    for (int tg = 0; tg < TG; tg++)
+                        acc[tg][e & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[tg][e], bv, acc[tg][e & 1], 0, 0, 0);
+                }
+            }
+        };
+        // grad_input of one channel: K * V fused multiply-adds with the channel's weights
+        // (wave-uniform: scalar loads into scalar registers), then the store
+        auto load_weights = [&](int ci, float (&w)[K]) {
+            const float *kc = kw + (int64_t)ci * K;
+#pragma unroll
+            for (int t = 0; t < K; t++) w[t] = kc[t];
+        };
+        // `prefetch`: the weights of the next channel are requested right after the first use
+        // of this channel's (scalar loads return in any order, so only a wait for all of them
+        // exists: the request must follow that wait to have the rest of the arithmetic to land in)
+        auto update_channel = [&](int ci, float (&gv)[V], const float (&w)[K], auto prefetch, float (&wn)[K]) {
+            float sum[V];
+#pragma unroll
+            for (int i = 0; i < V; i++) sum[i] = w[0] * tv[0][i];
+            __builtin_amdgcn_sched_barrier(0);
+            if (decltype(prefetch)::value) load_weights(ci + 1, wn);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int t = 1; t < K; t++)
+#pragma unroll
+                for (int i = 0; i < V; i++) sum[i] += w[t] * tv[t][i];
+#pragma unroll
+            for (int i = 0; i < V; i++) gv[i] += sum[i];
+            store_vec<V>(reinterpret_cast<float *>(gbase + (int64_t)ci * gsc * 4 + goff), gv);
+        };
+        // grad_input of one stage: up to NCS channels.  Lanes past the row sit the whole stage
+        // out, so that the channels form one straight run of code.
+        auto stage_x = [&](int cb, int h, float (&gg)[NCS][V]) {
+            const int cj0 = c0 + cb * kChanBlock + h * NCS;
+            if (!act) return;
+            float w[2][K];
+            if (cj0 + NCS <= cx_end) {            // uniform: all channels of the stage exist
+                load_weights(cj0, w[0]);
+#pragma unroll
+                for (int j = 0; j < NCS; j++) {
+                    if (j + 1 < NCS)
+                        update_channel(cj0 + j, gg[j], w[j & 1], std::true_type{}, w[(j + 1) & 1]);
+                    else
+                        update_channel(cj0 + j, gg[j], w[j & 1], std::false_type{}, w[(j + 1) & 1]);
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < NCS; j++)
+                    if (cj0 + j < cx_end) {
+                        load_weights(cj0 + j, w[0]);
+                        update_channel(cj0 + j, gg[j], w[0], std::false_type{}, w[1]);
+                    }
+            }
+        };
+
+        // ---- channel loop: blocks of 16 channels, H stages each, two stages per iteration; the
+        // loads of the next stage are issued before the arithmetic of the current one
+        const int nst = ncb * H;                  // even
+#pragma unroll 1
+        for (int st = 0; st < nst; st += 2) {
+            const int cb = st / H, h = st % H;
+            load_stage(cb, h + 1, kb, gb);
+#pragma unroll
+            for (int tg = 0; tg < TG; tg++) acc[tg][0] = acc[tg][1] = mfma4{0.f, 0.f, 0.f, 0.f};
+            stage_k(cb, h, ka);
+            stage_x(cb, h, ga);
+            if (st + 2 < nst) load_stage((st + 2) / H, (st + 2) % H, ka, ga);
+            stage_k(cb, h + 1, kb);
+            stage_x(cb, h + 1, gb);
+            // D is indexed statically: pick the block with a chain of uniform branches
+#pragma unroll
+            for (int q = 0; q < NCB; q++)
+                if (q == cb) {
+#pragma unroll
+                    for (int tg = 0; tg < TG; tg++) D[q][tg] += acc[tg][0] + acc[tg][1];
+                }
+        }
+        // Channels from mask_from on are outputs of the layer below: their gradient is complete
+        // with this update, so its ReLU mask is applied now (every lane revisits what it wrote).
+        if (act) {
+            for (int ci = max(a.mask_from, c0); ci < cx_end; ci++) {
+                float m[V], v[V];
+                float *gpc = reinterpret_cast<float *>(gbase + (int64_t)ci * gsc * 4 + goff);
+                load_vec<V>(reinterpret_cast<const float *>(abase + (int64_t)ci * gsc * 4 + goff), m);
+                load_vec<V>(gpc, v);
+#pragma unroll
+                for (int i = 0; i < V; i++) v[i] = 0.f < m[i] ? v[i] : 0.f;
+                store_vec<V>(gpc, v);
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+
+    // D[cb][tg][v] = sum for tap tg*16 + 4*mk + v, channel c0 + cb*16 + mj.  Add the waves in LDS.
+    __syncthreads();
+    constexpr int PER_WAVE = NCB * TG * 4 * kWave;
+    float *red = lds;
+#pragma unroll
+    for (int cb = 0; cb < NCB; cb++)
+#pragma unroll
+        for (int tg = 0; tg < TG; tg++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) red[wave * PER_WAVE + ((cb * TG + tg) * 4 + v) * kWave + wl] = D[cb][tg][v];
+    __syncthreads();
+    // partial sums are stored column-major, part[column][workgroup], so that the
+    // second pass reads each column as one contiguous run
+    float *pcol = part + blockIdx.x;
+    for (int idx = tid; idx < PER_WAVE; idx += blockDim.x) {
+        const int l = idx % kWave, v = (idx / kWave) % 4, tg = (idx / (4 * kWave)) % TG, cb = idx / (4 * kWave * TG);
+        const int tap = tg * 16 + 4 * (l / 16) + v;
+        const int ch = c0 + cb * kChanBlock + l % 16;
+        if (tap >= K || ch >= c_end) continue;
+        float s = 0.f;
+        for (int w = 0; w < nwaves; w++) s += red[w * PER_WAVE + idx];
+        if (ch < g.C)
+            pcol[((int64_t)ch * K + tap) * kMaxPartialRows] = s;
+        else if (tap == K / 2)
+            pcol[((int64_t)g.C * K) * kMaxPartialRows] = s;
+    }
+}
+
+template <int NDIM, int V, int NCB>
+size_t lds_bytes(const RowTeams &rt)
+{
+    constexpr int TG = NDIM == 3 ? 2 : 1;
+    const size_t main_loop =
+        ((size_t)rt.rpw * RowTaps<NDIM>::NPQ * V * rt.lpr + (size_t)kWaves * ATile<NDIM, V>::kFloats) * 4;
+    const size_t epilogue = (size_t)kWaves * NCB * TG * 4 * kWave * 4;
+    return std::max(main_loop, epilogue);
+}
+
+// Strides and in-plane offsets fit the kernel's 32-bit arithmetic.
+template <typename T>
+inline bool small_strides(const Geom &g, const View<T> &v)
+{
+    const int64_t lim = (int64_t)1 << 30;
+    if (v.sb >= lim * 2 || v.sc >= lim * 2 || v.sz >= lim || v.sy >= lim) return false;
+    return (int64_t)(g.D - 1) * v.sz + (int64_t)(g.H - 1) * v.sy + g.W < lim;
+}
+
+// Usable with V voxels per lane: whole waves per row, rows fit a 256-lane workgroup,
+// 16-byte accesses to x and V-wide ones to the other tensors aligned.
+template <int NDIM>
+bool fits(const Geom &g, int V, const View<const float> &gy, const View<const float> &x, const View<float> &gx)
+{
+    RowTeams rt;
+    if (g.W % 4 != 0 || !make_row_teams(g, V, &rt)) return false;
+    if (rt.lpr % kWave != 0 || rt.lpr * rt.rpw > kThreads) return false;
+    return rows_aligned(x, g.W, 4) && rows_aligned(gy, g.W, V) && rows_aligned(gx, g.W, V);
+}
+
+template <int NDIM>
+int choose_vec(const Geom &g, int vmax, const View<const float> &gy, const View<const float> &x,
+               const View<float> &gx)
+{
+    for (int v = NDIM == 3 ? 2 : 4; v >= 1; v /= 2) {
+        if (v > vmax) continue;
+        if (fits<NDIM>(g, v, gy, x, gx)) return v;
+    }
+    return 0;
+}
+
+template <int NDIM, int V, int NCB>
+hipError_t launch(const Geom &g, const View<const float> &gy, const View<const float> &x, const float *k,
+                  const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws, hipStream_t s)
+{
+    constexpr int K = Taps<NDIM>::K;
+    Args a;
+    a.g = g;
+    make_row_teams(g, V, &a.rt);
+    float *part = ws + backward_k_mask_floats(g);
+    a.ngroups = (a.rt.nrows + a.rt.rpw - 1) / a.rt.rpw;
+    const int64_t total = (int64_t)a.ngroups * g.B;
+    a.remap = knob(kKnobXcdRemap, 1);
+    const int64_t max_wgs = std::min<int64_t>(std::max(8, knob(kKnobBwdkBlocks, kMaxPartialRows)), kMaxPartialRows);
+    a.tiles_per_wg = (int)((total + max_wgs - 1) / max_wgs);
+    const int64_t wgs = (total + a.tiles_per_wg - 1) / a.tiles_per_wg;
+    const int rows = a.remap ? xcd_grid((int)wgs) : (int)wgs;   // padding workgroups write zero rows
+    if (rows > kMaxPartialRows || total > INT32_MAX) return hipErrorInvalidConfiguration;
+    a.total_groups = (int)total;
+    a.gy = Plane{(int)gy.sb, (int)gy.sc, (int)gy.sz, (int)gy.sy};
+    a.x = Plane{(int)x.sb, (int)x.sc, (int)x.sz, (int)x.sy};
+    a.gx = Plane{(int)gx.sb, (int)gx.sc, (int)gx.sz, (int)gx.sy};
+    const float *actp = pm.from < g.C ? pm.act.p : x.p;   // only dereferenced for channels >= mask_from
+    a.mask_from = pm.from;
+    a.want_bias = gb != nullptr;
+    const int chunks = (g.C + a.want_bias + NCB * kChanBlock - 1) / (NCB * kChanBlock);
+    const size_t lds = lds_bytes<NDIM, V, NCB>(a.rt);
+    hipLaunchKernelGGL((bwd_rows_fused<NDIM, V, NCB>), dim3(rows, 1, chunks), dim3(a.rt.lpr * a.rt.rpw), lds, s, a,
+                       gy.p, x.p, gx.p, actp, k, part);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    const int64_t nk = (int64_t)g.C * K;
+    const int64_t ncols = nk + (a.want_bias ? 1 : 0);
+    hipLaunchKernelGGL(bwdk::reduce_columns, dim3((ncols + 3) / 4), dim3(256), 0, s, part, rows, nk, ncols, gk, gb);
+    return hipGetLastError();
+}
+
+template <int NDIM, int V>
+hipError_t pick_ncb(const Geom &g, const View<const float> &gy, const View<const float> &x, const float *k,
+                    const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws, hipStream_t s)
+{
+    const int need = (g.C + (gb != nullptr) + kChanBlock - 1) / kChanBlock;
+    if (need <= 1) return launch<NDIM, V, 1>(g, gy, x, k, gx, pm, gk, gb, ws, s);
+    if (need <= 2) return launch<NDIM, V, 2>(g, gy, x, k, gx, pm, gk, gb, ws, s);
+    if (need <= 4) return launch<NDIM, V, 4>(g, gy, x, k, gx, pm, gk, gb, ws, s);
+    return launch<NDIM, V, 8>(g, gy, x, k, gx, pm, gk, gb, ws, s);
+}
+
+// One output channel, unit x-strides, 32-bit strides, and a vector width that fits.
+template <int NDIM>
+bool xkb_supported_nd(const Geom &g, const View<const float> &gy, const View<const float> &x, const View<float> &gx)
+{
+    if (g.Wd != 1 || x.sx != 1 || gy.sx != 1 || gx.sx != 1) return false;
+    if (!small_strides(g, gy) || !small_strides(g, x) || !small_strides(g, gx)) return false;
+    return choose_vec<NDIM>(g, 4, gy, x, gx) != 0;
+}
+
+// pm.act, where pm.from < C, must be laid out like gx (same strides and 16-byte phase).
+template <int NDIM>
+hipError_t xkb_nd(const Geom &g, const View<const float> &gy, const View<const float> &x, const float *k,
+                  const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws, hipStream_t s)
+{
+    const int vmax = knob(NDIM == 3 ? kKnobBwdkVec3d : kKnobBwdkVec2d, 4);
+    int v = choose_vec<NDIM>(g, vmax, gy, x, gx);
+    if (v == 0) v = choose_vec<NDIM>(g, 4, gy, x, gx);
+    if constexpr (NDIM == 2) {
+        if (v == 4) return pick_ncb<2, 4>(g, gy, x, k, gx, pm, gk, gb, ws, s);
+    }
+    if (v == 2) return pick_ncb<NDIM, 2>(g, gy, x, k, gx, pm, gk, gb, ws, s);
+    if (v == 1) return pick_ncb<NDIM, 1>(g, gy, x, k, gx, pm, gk, gb, ws, s);
+    return hipErrorInvalidConfiguration;
+}
+
+}  // namespace bwdxk
+}  // namespace msd

@@ -38,7 +38,7 @@ hipError_t generic_backward_kb(const Geom &g, bool relu, View<const T> out, View
 enum Knob {
     kKnobBwdxVec2d, kKnobBwdxVec3d, kKnobBwdxUnroll2d, kKnobBwdxUnroll3d, kKnobBwdxMinBlocks,
     kKnobXcdRemap, kKnobBwdkVec2d, kKnobBwdkVec3d, kKnobBwdkBlocks,
-    kKnobFwdVec2d, kKnobFwdVec3d, kKnobFwdSplit, kKnobFwdRows2d, kKnobBwdkRows,
+    kKnobFwdVec2d, kKnobFwdVec3d, kKnobFwdSplit, kKnobFwdRows2d, kKnobBwdkRows, kKnobBlockFuse,
     kKnobCount
 };
 int knob(Knob k, int dflt);
@@ -117,6 +117,33 @@ inline hipError_t fast_backward_kb(const Geom &g, bool relu, const View<const fl
 {
     return g.ndim == 3 ? fast_backward_kb_3d(g, relu, out, gy, x, gk, gb, ws, s)
                        : fast_backward_kb_2d(g, relu, out, gy, x, gk, gb, ws, s);
+}
+
+// backward_x and backward_k (+ bias) of one layer in one pass (one output channel, the
+// ReLU mask already applied to gy); gk must not be null, gb may be.  Same workspace as
+// fast_backward_kb.
+bool fast_backward_xkb_supported_2d(const Geom &g, const View<const float> &gy, const View<const float> &x,
+                                    const View<float> &gx);
+bool fast_backward_xkb_supported_3d(const Geom &g, const View<const float> &gy, const View<const float> &x,
+                                    const View<float> &gx);
+hipError_t fast_backward_xkb_2d(const Geom &g, const View<const float> &gy, const View<const float> &x, const float *k,
+                                const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws,
+                                hipStream_t s);
+hipError_t fast_backward_xkb_3d(const Geom &g, const View<const float> &gy, const View<const float> &x, const float *k,
+                                const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws,
+                                hipStream_t s);
+
+inline bool fast_backward_xkb_supported(const Geom &g, const View<const float> &gy, const View<const float> &x,
+                                        const View<float> &gx)
+{
+    return g.ndim == 3 ? fast_backward_xkb_supported_3d(g, gy, x, gx) : fast_backward_xkb_supported_2d(g, gy, x, gx);
+}
+inline hipError_t fast_backward_xkb(const Geom &g, const View<const float> &gy, const View<const float> &x,
+                                    const float *k, const View<float> &gx, const PostMask &pm, float *gk, float *gb,
+                                    float *ws, hipStream_t s)
+{
+    return g.ndim == 3 ? fast_backward_xkb_3d(g, gy, x, k, gx, pm, gk, gb, ws, s)
+                       : fast_backward_xkb_2d(g, gy, x, k, gx, pm, gk, gb, ws, s);
 }
 
 }  // namespace msd
