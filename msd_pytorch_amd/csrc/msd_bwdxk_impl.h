@@ -384,7 +384,8 @@ hipError_t launch(const Geom &g, const View<const float> &gy, const View<const f
     a.ngroups = (a.rt.nrows + a.rt.rpw - 1) / a.rt.rpw;
     const int64_t total = (int64_t)a.ngroups * g.B;
     a.remap = knob(kKnobXcdRemap, 1);
-    const int64_t max_wgs = std::min<int64_t>(std::max(8, knob(kKnobBwdkBlocks, kMaxPartialRows)), kMaxPartialRows);
+    // two workgroups per CU are resident (registers): with that many the grid runs as one round
+    const int64_t max_wgs = std::min<int64_t>(std::max(8, knob(kKnobBwdkBlocks, 512)), kMaxPartialRows);
     a.tiles_per_wg = (int)((total + max_wgs - 1) / max_wgs);
     const int64_t wgs = (total + a.tiles_per_wg - 1) / a.tiles_per_wg;
     const int rows = a.remap ? xcd_grid((int)wgs) : (int)wgs;   // padding workgroups write zero rows
@@ -433,7 +434,8 @@ template <int NDIM>
 hipError_t xkb_nd(const Geom &g, const View<const float> &gy, const View<const float> &x, const float *k,
                   const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws, hipStream_t s)
 {
-    const int vmax = knob(NDIM == 3 ? kKnobBwdkVec3d : kKnobBwdkVec2d, 4);
+    // 3D: one voxel per lane keeps the 27 gathered values per voxel and the pipeline buffers in registers
+    const int vmax = knob(NDIM == 3 ? kKnobBwdkVec3d : kKnobBwdkVec2d, NDIM == 3 ? 1 : 4);
     int v = choose_vec<NDIM>(g, vmax, gy, x, gx);
     if (v == 0) v = choose_vec<NDIM>(g, 4, gy, x, gx);
     if constexpr (NDIM == 2) {

@@ -55,6 +55,50 @@ def test_block_matches_oracle(ndim, size, c_in, width, depth, dtype):
         assert rel_err(a.grad, b) <= tg
 
 
+@pytest.mark.parametrize("ndim,size,c_in,depth,batch,dilations", [
+    # shapes the fused backward_x + backward_k kernel of the block takes (width 1, rows of
+    # whole 4-voxel groups and at least one wavefront), with ragged rows, row groups and
+    # channel blocks (16 input channels each, plus the bias column)
+    (2, (37, 256), 1, 20, 2, None),        # 4 voxels per lane, 4 rows per workgroup, 37 rows
+    (2, (9, 1024), 2, 5, 1, None),         # one row per workgroup
+    (2, (30, 132), 3, 36, 1, None),        # 33 of 64 lanes per row busy; 3 channel blocks
+    (2, (40, 128), 1, 4, 1, [1, 7, 31, 40]),   # dilations up to the image height
+    (3, (9, 11, 128), 1, 18, 1, None),     # one voxel per lane, 2 rows per workgroup
+    (3, (6, 7, 68), 2, 6, 2, None),        # 68 of 128 lanes per row busy
+    (3, (12, 5, 64), 1, 3, 1, [5, 1, 4]),  # dilation == smallest extent
+])
+def test_fused_block_backward_matches_oracle(ndim, size, c_in, depth, batch, dilations):
+    from msd_pytorch_amd import _native
+    from msd_pytorch_amd.msd_block import msd_block
+    x, dil, bias, ws, g = make_block_problem(ndim, size, c_in, 1, depth, torch.float32, batch=batch)
+    if dilations is not None:
+        dil = dilations
+    want = oracle.block_forward(x.double(), dil, bias.double(), [w.double() for w in ws])
+    want_gx, want_gb, want_gw = oracle.block_backward(want, g.double(), dil, bias.double(), [w.double() for w in ws])
+
+    lib = _native.load()
+    results = {}
+    for fuse in (1, 0):
+        assert lib.msd_set_tuning(b"block.fuse", fuse) == 0
+        try:
+            xd = x.cuda().requires_grad_(True)
+            bd = bias.cuda().requires_grad_(True)
+            wd = [w.cuda().requires_grad_(True) for w in ws]
+            got = msd_block(xd, dil, bd, *wd)
+            got.backward(g.cuda())
+            torch.cuda.synchronize()
+        finally:
+            lib.msd_set_tuning(b"block.fuse", -1)
+        assert rel_err(got, want) <= 1e-5
+        assert rel_err(xd.grad, want_gx) <= 1e-4
+        assert rel_err(bd.grad, want_gb) <= 1e-4
+        assert max(rel_err(a.grad, b) for a, b in zip(wd, want_gw)) <= 1e-4
+        results[fuse] = (xd.grad, bd.grad, [w.grad for w in wd])
+    # the fused and the separate kernels add the same terms in different orders
+    assert rel_err(results[1][0], results[0][0]) <= 1e-5
+    assert max(rel_err(a, b) for a, b in zip(results[1][2], results[0][2])) <= 1e-5
+
+
 def test_depth_100_stack_stays_within_tolerance():
     # errors compound through the layers: the full depth of the headline network on a small image
     from msd_pytorch_amd.msd_block import msd_block
