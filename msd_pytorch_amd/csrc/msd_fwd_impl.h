@@ -28,6 +28,8 @@
 namespace msd {
 namespace fwd {
 
+constexpr int kOrder = 4;   // edge of the (y, z) blocks the 3D tiles are numbered in
+
 struct Lattice {
     int lpr;        // lanes per row
     int ks;         // channel groups per workgroup
@@ -52,7 +54,20 @@ __global__ __launch_bounds__(1024) void fwd_lattice(Geom g, Lattice lt, int rema
 
     const int tile = block_for_xcd(blockIdx.x, gridDim.x, remap);
     if (tile >= lt.ntiles) return;               // padding block
-    const int ty = tile % lt.tiles_y, tz = tile / lt.tiles_y;
+    // 3D: tiles are numbered in blocks of kOrder x kOrder (y, z) neighbours.  Neighbouring
+    // lattices share a third of their input rows, and only tiles that start together walk the
+    // channels in step and find each other's rows in the L2.
+    int ty, tz;
+    if (NDIM == 3) {
+        const int blk = tile / (kOrder * kOrder), within = tile % (kOrder * kOrder);
+        const int nby = (lt.tiles_y + kOrder - 1) / kOrder;
+        ty = (blk % nby) * kOrder + within % kOrder;
+        tz = (blk / nby) * kOrder + within / kOrder;
+        if (ty >= lt.tiles_y || tz >= lt.tiles_z) return;   // padding of the block grid (whole workgroup)
+    } else {
+        ty = tile;
+        tz = 0;
+    }
     const int y0 = ty / lt.segs_y + (ty % lt.segs_y) * RY * g.dil;
     const int z0 = NDIM == 3 ? tz / lt.segs_z + (tz % lt.segs_z) * RZ * g.dil : 0;
     if (y0 >= g.H || z0 >= g.D) return;          // empty tail of a residue class (whole workgroup)
@@ -63,15 +78,18 @@ __global__ __launch_bounds__(1024) void fwd_lattice(Geom g, Lattice lt, int rema
     const bool act = lane * V < g.W;
     const int b = blockIdx.y;
 
-    // element offsets of the input lattice rows (fold, then clamp rows that only
-    // feed output rows outside the image)
-    int64_t offz[LZ], offy[LY];
+    // Offsets of the input lattice rows (fold, then clamp rows that only feed output rows
+    // outside the image).  A load address is a wave-uniform base (batch, channel, z level:
+    // scalar registers and scalar arithmetic) plus a 32-bit byte offset per lane (y row and
+    // x position, computed once), so the channel loop spends no vector instructions on it.
+    int64_t offz[LZ];
+    uint32_t offyx[LY];
 #pragma unroll
     for (int m = 0; m < LZ; m++)
-        offz[m] = NDIM == 3 ? (int64_t)min(reflect_idx(min(z0 + (m - 1) * g.dil, 2 * g.D - 1), g.D), g.D - 1) * x.sz : 0;
+        offz[m] = NDIM == 3 ? (int64_t)min(reflect_idx(min(z0 + (m - 1) * g.dil, 2 * g.D - 1), g.D), g.D - 1) * x.sz * 4 : 0;
 #pragma unroll
     for (int m = 0; m < LY; m++)
-        offy[m] = (int64_t)min(reflect_idx(min(y0 + (m - 1) * g.dil, 2 * g.H - 1), g.H), g.H - 1) * x.sy;
+        offyx[m] = 4u * (uint32_t)(min(reflect_idx(min(y0 + (m - 1) * g.dil, 2 * g.H - 1), g.H), g.H - 1) * (int)x.sy + x0);
 
     // valid output rows of this lattice (the rest lie past the image edge)
     const int nyv = min(RY, (g.H - y0 + g.dil - 1) / g.dil);
@@ -89,20 +107,28 @@ __global__ __launch_bounds__(1024) void fwd_lattice(Geom g, Lattice lt, int rema
 #pragma unroll
                     for (int i = 0; i < V; i++) acc[co][jz][jy][r][i] = 0.f;
 
-    const float *xb = x.p + (int64_t)b * x.sb + x0;
+    const char *xb = reinterpret_cast<const char *>(x.p + (int64_t)b * x.sb);
     for (int ci = kg; ci < g.C; ci += lt.ks) {
-        const float *xc = xb + (int64_t)ci * x.sc;
+        const char *xc = xb + (int64_t)ci * x.sc * 4;
         float w[WOUT][K];
 #pragma unroll
         for (int co = 0; co < WOUT; co++)
 #pragma unroll
             for (int t = 0; t < K; t++) w[co][t] = k[((int64_t)co * g.C + ci) * K + t];
+        // (redefining the lane offsets here keeps their widening to 64 bits inside the loop, next
+        // to the loads, where it costs nothing; hoisted, it would turn them into register pairs
+        // and every load address into a 64-bit vector addition)
+#pragma unroll
+        for (int my = 0; my < LY; my++) asm volatile("" : "+v"(offyx[my]));
         // all row loads of this channel are issued before the first multiply-add
         float xv[LZ][LY][V];
 #pragma unroll
-        for (int mz = 0; mz < LZ; mz++)
+        for (int mz = 0; mz < LZ; mz++) {
+            uint64_t xz = reinterpret_cast<uint64_t>(xc + offz[mz]);
+            asm volatile("" : "+s"(xz));          // stays a scalar base: the loads take it beside the lane offset
 #pragma unroll
-            for (int my = 0; my < LY; my++) load_vec<V>(xc + offz[mz] + offy[my], xv[mz][my]);
+            for (int my = 0; my < LY; my++) load_global_vec<V>(xz, offyx[my], xv[mz][my]);
+        }
         if constexpr (WOUT == 1) __builtin_amdgcn_sched_barrier(0);
         // output rows past the image edge (partial lattices) are skipped, uniformly per workgroup
 #pragma unroll
@@ -191,11 +217,12 @@ inline bool make_lattice(const Geom &g, int V, int rz, int ry, int ks_wanted, La
     if (g.ndim == 3) {
         lt->segs_z = ((g.D + g.dil - 1) / g.dil + rz - 1) / rz;
         lt->tiles_z = g.dil * lt->segs_z;
+        lt->ntiles = ((lt->tiles_y + kOrder - 1) / kOrder) * ((lt->tiles_z + kOrder - 1) / kOrder) * kOrder * kOrder;
     } else {
         lt->segs_z = 1;
         lt->tiles_z = 1;
+        lt->ntiles = lt->tiles_y;
     }
-    lt->ntiles = lt->tiles_y * lt->tiles_z;
     return true;
 }
 
@@ -231,6 +258,7 @@ template <int NDIM>
 bool supported_nd(const Geom &g, const View<const float> &x, const View<float> &out)
 {
     if (g.Wd > 2 || x.sx != 1 || out.sx != 1) return false;
+    if ((int64_t)(g.H - 1) * x.sy + g.W >= ((int64_t)1 << 30)) return false;   // 32-bit in-plane byte offsets
     if (g.W < 32) return false;                  // rows shorter than half a wave: the generic kernel does better
     return choose_vec(g, 4, x, out) != 0;
 }

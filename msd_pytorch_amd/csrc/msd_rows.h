@@ -66,6 +66,22 @@ template <> __device__ __forceinline__ void load_vec<4>(const float *p, float (&
     const f32x4 v = *reinterpret_cast<const f32x4 *>(p);
     d[0] = v[0]; d[1] = v[1]; d[2] = v[2]; d[3] = v[3];
 }
+// The same from global memory at a wave-uniform 64-bit base plus a 32-bit byte offset per
+// lane: the form the load instruction takes directly (scalar base, vector offset).
+template <int V>
+__device__ __forceinline__ void load_global_vec(uint64_t base, uint32_t byte_offset, float (&d)[V])
+{
+    typedef const __attribute__((address_space(1))) char *gbytes_t;
+    gbytes_t p = reinterpret_cast<gbytes_t>(base) + byte_offset;
+    if constexpr (V == 1) {
+        d[0] = *reinterpret_cast<const __attribute__((address_space(1))) float *>(p);
+    } else {
+        typedef float vec_t __attribute__((ext_vector_type(V)));
+        const vec_t v = *reinterpret_cast<const __attribute__((address_space(1))) vec_t *>(p);
+#pragma unroll
+        for (int i = 0; i < V; i++) d[i] = v[i];
+    }
+}
 template <int V> __device__ __forceinline__ void store_vec(float *p, const float (&d)[V]);
 template <> __device__ __forceinline__ void store_vec<1>(float *p, const float (&d)[1]) { *p = d[0]; }
 template <> __device__ __forceinline__ void store_vec<2>(float *p, const float (&d)[2])
