@@ -122,12 +122,20 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_rows_fused(const Args a, cons
         const bool act = rowok && x0 < g.W;
         const int rr = min(row, rt.nrows - 1);
         const int y = rr % g.H, z = rr / g.H;
-        // x: per-lane channel, so a full address per lane
-        const float *xk = xp + (int64_t)b * a.x.sb + (int64_t)z * a.x.sz + (int64_t)y * a.x.sy;
-        // grad_input and activations: uniform base of (batch, channel) + byte offset of the lane's voxels
-        char *gbase = reinterpret_cast<char *>(gxp + (int64_t)b * a.gx.sb);
-        const char *abase = reinterpret_cast<const char *>(actp + (int64_t)b * a.gx.sb);
-        const uint32_t goff = 4u * (uint32_t)(z * a.gx.sz + y * a.gx.sy + xc);
+        // Addresses are a wave-uniform 64-bit base (scalar registers) plus a 32-bit byte offset
+        // per lane, the form the memory instructions take directly.  x: the lane's channel is
+        // part of the offset; grad_input and activations: the channel is part of the base.
+        const uint64_t xbase = reinterpret_cast<uint64_t>(xp + (int64_t)b * a.x.sb);
+        const uint32_t xrow = (uint32_t)(z * a.x.sz + y * a.x.sy);
+        const uint64_t gbase = reinterpret_cast<uint64_t>(gxp + (int64_t)b * a.gx.sb);
+        const uint64_t abase = reinterpret_cast<uint64_t>(actp + (int64_t)b * a.gx.sb);
+        uint32_t goff = 4u * (uint32_t)(z * a.gx.sz + y * a.gx.sy + xc);
+        // uniform base of grad_input channel ci, kept in scalar registers
+        auto channel_base = [&](uint64_t base, int ci) {
+            uint64_t p = base + (uint64_t)((int64_t)ci * gsc * 4);
+            asm volatile("" : "+s"(p));
+            return p;
+        };
 
         // ---- one pipeline stage of loads: NSS 16-voxel groups of 16 channels of x in the MFMA B
         // layout, and NCS channels of grad_input in the voxel layout.  Clamped, always valid
@@ -135,17 +143,17 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_rows_fused(const Args a, cons
         float ka[NSS][4], kb[NSS][4];             // stages alternate between the a and b buffers
         float ga[NCS][V], gb[NCS][V];
         auto load_stage = [&](int cb, int h, float (&kk)[NSS][4], float (&gg)[NCS][V]) {
-            const float *p = xk + (int64_t)min(c0 + cb * kChanBlock + mj, g.C - 1) * xsc;
+            // (redefining the lane offset keeps its widening to 64 bits next to the loads, where
+            // it is free; hoisted out of the loop it would make every address a vector addition)
+            asm volatile("" : "+v"(goff));
+            const uint32_t xch = (uint32_t)min(c0 + cb * kChanBlock + mj, g.C - 1) * (uint32_t)xsc + xrow;
 #pragma unroll
-            for (int j = 0; j < NSS; j++) {
-                const f32x4 v = *reinterpret_cast<const f32x4 *>(p + min(kx + 16 * (h * NSS + j), g.W - 4));
-#pragma unroll
-                for (int e = 0; e < 4; e++) kk[j][e] = v[e];
-            }
+            for (int j = 0; j < NSS; j++)
+                load_global_vec<4>(xbase, 4u * (xch + (uint32_t)min(kx + 16 * (h * NSS + j), g.W - 4)), kk[j]);
 #pragma unroll
             for (int j = 0; j < NCS; j++) {
                 const int ci = max(min(c0 + cb * kChanBlock + h * NCS + j, cx_end - 1), 0);
-                load_vec<V>(reinterpret_cast<const float *>(gbase + (int64_t)ci * gsc * 4 + goff), gg[j]);
+                load_global_vec<V>(channel_base(gbase, ci), goff, gg[j]);
             }
         };
         load_stage(0, 0, ka, ga);   // issued ahead of the gather so the two latencies overlap
@@ -236,13 +244,14 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_rows_fused(const Args a, cons
                 for (int i = 0; i < V; i++) sum[i] += w[t] * tv[t][i];
 #pragma unroll
             for (int i = 0; i < V; i++) gv[i] += sum[i];
-            store_vec<V>(reinterpret_cast<float *>(gbase + (int64_t)ci * gsc * 4 + goff), gv);
+            store_global_vec<V>(channel_base(gbase, ci), goff, gv);
         };
         // grad_input of one stage: up to NCS channels.  Lanes past the row sit the whole stage
         // out, so that the channels form one straight run of code.
         auto stage_x = [&](int cb, int h, float (&gg)[NCS][V]) {
             const int cj0 = c0 + cb * kChanBlock + h * NCS;
             if (!act) return;
+            asm volatile("" : "+v"(goff));        // as in load_stage: the stores take base + lane offset directly
             float w[2][K];
             if (cj0 + NCS <= cx_end) {            // uniform: all channels of the stage exist
                 load_weights(cj0, w[0]);
@@ -290,12 +299,11 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_rows_fused(const Args a, cons
         if (act) {
             for (int ci = max(a.mask_from, c0); ci < cx_end; ci++) {
                 float m[V], v[V];
-                float *gpc = reinterpret_cast<float *>(gbase + (int64_t)ci * gsc * 4 + goff);
-                load_vec<V>(reinterpret_cast<const float *>(abase + (int64_t)ci * gsc * 4 + goff), m);
-                load_vec<V>(gpc, v);
+                load_global_vec<V>(channel_base(abase, ci), goff, m);
+                load_global_vec<V>(channel_base(gbase, ci), goff, v);
 #pragma unroll
                 for (int i = 0; i < V; i++) v[i] = 0.f < m[i] ? v[i] : 0.f;
-                store_vec<V>(gpc, v);
+                store_global_vec<V>(channel_base(gbase, ci), goff, v);
             }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -426,6 +434,7 @@ bool xkb_supported_nd(const Geom &g, const View<const float> &gy, const View<con
 {
     if (g.Wd != 1 || x.sx != 1 || gy.sx != 1 || gx.sx != 1) return false;
     if (!small_strides(g, gy) || !small_strides(g, x) || !small_strides(g, gx)) return false;
+    if ((int64_t)g.C * x.sc + (int64_t)g.D * x.sz + (int64_t)g.H * x.sy + g.W >= ((int64_t)1 << 30)) return false;
     return choose_vec<NDIM>(g, 4, gy, x, gx) != 0;
 }
 

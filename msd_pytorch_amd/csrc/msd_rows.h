@@ -82,6 +82,21 @@ __device__ __forceinline__ void load_global_vec(uint64_t base, uint32_t byte_off
         for (int i = 0; i < V; i++) d[i] = v[i];
     }
 }
+template <int V>
+__device__ __forceinline__ void store_global_vec(uint64_t base, uint32_t byte_offset, const float (&d)[V])
+{
+    typedef __attribute__((address_space(1))) char *gbytes_t;
+    gbytes_t p = reinterpret_cast<gbytes_t>(base) + byte_offset;
+    if constexpr (V == 1) {
+        *reinterpret_cast<__attribute__((address_space(1))) float *>(p) = d[0];
+    } else {
+        typedef float vec_t __attribute__((ext_vector_type(V)));
+        vec_t v;
+#pragma unroll
+        for (int i = 0; i < V; i++) v[i] = d[i];
+        *reinterpret_cast<__attribute__((address_space(1))) vec_t *>(p) = v;
+    }
+}
 template <int V> __device__ __forceinline__ void store_vec(float *p, const float (&d)[V]);
 template <> __device__ __forceinline__ void store_vec<1>(float *p, const float (&d)[1]) { *p = d[0]; }
 template <> __device__ __forceinline__ void store_vec<2>(float *p, const float (&d)[2])
