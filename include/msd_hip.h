@@ -217,6 +217,29 @@ int msd_block_backward(int dtype, int ndim, int64_t batch, int64_t c_in, int dep
                        void *workspace, int64_t workspace_bytes, void *stream);
 
 /*
+ * Final layer of the network: out[b][o][n] = bias[o] + sum_c weight[o][c] * input[b][c][n],
+ * the Conv1d(c_in, c_out, 1) over the flattened voxels of MSDFinalLayer
+ * (msd_module.py:60-88), which the reference leaves to torch.  `nvox` voxels per channel
+ * are contiguous; batch and channel strides are in elements, so `input` can be the dense
+ * block's stack as it is.  weight is contiguous (c_out, c_in), bias (c_out) or NULL.
+ * msd_final_backward OVERWRITES grad_input (same layout rules; NULL to skip),
+ * grad_weight and grad_bias (either may be NULL); the sums over voxels are reduced in a
+ * fixed order through `workspace` (msd_final_workspace_bytes).
+ */
+int64_t msd_final_workspace_bytes(int dtype, int64_t batch, int64_t c_in, int64_t c_out, int64_t nvox);
+int msd_final_forward(int dtype, int64_t batch, int64_t c_in, int64_t c_out, int64_t nvox,
+                      const void *input, int64_t input_batch_stride, int64_t input_channel_stride,
+                      const void *weight, const void *bias,
+                      void *output, int64_t output_batch_stride, int64_t output_channel_stride, void *stream);
+int msd_final_backward(int dtype, int64_t batch, int64_t c_in, int64_t c_out, int64_t nvox,
+                       const void *input, int64_t input_batch_stride, int64_t input_channel_stride,
+                       const void *grad_output, int64_t grad_output_batch_stride, int64_t grad_output_channel_stride,
+                       const void *weight,
+                       void *grad_input, int64_t grad_input_batch_stride, int64_t grad_input_channel_stride,
+                       void *grad_weight, void *grad_bias,
+                       void *workspace, int64_t workspace_bytes, void *stream);
+
+/*
  * Kernel timing for benchmarks.  While enabled, every operator call (also inside
  * the block calls) is bracketed by HIP events recorded on its launch stream.
  * msd_profile_read waits for the recorded events and returns, per class

@@ -46,6 +46,11 @@ PROTOTYPES = {
     "msd_block_backward": (_c_int, [_c_int, _c_int, _c_i64, _c_i64, _c_int, _i64p, _i64p, _i64p] + _VIEW + _VIEW
                            + [ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ctypes.c_void_p), _ptr, _c_int]
                            + _WS + [_ptr]),
+    "msd_final_workspace_bytes": (_c_i64, [_c_int, _c_i64, _c_i64, _c_i64, _c_i64]),
+    "msd_final_forward": (_c_int, [_c_int, _c_i64, _c_i64, _c_i64, _c_i64, _ptr, _c_i64, _c_i64, _ptr, _ptr,
+                                   _ptr, _c_i64, _c_i64, _ptr]),
+    "msd_final_backward": (_c_int, [_c_int, _c_i64, _c_i64, _c_i64, _c_i64, _ptr, _c_i64, _c_i64, _ptr, _c_i64, _c_i64,
+                                    _ptr, _ptr, _c_i64, _c_i64, _ptr, _ptr] + _WS + [_ptr]),
     "msd_profile_enable": (_c_int, [_c_int]),
     "msd_profile_read": (_c_int, [ctypes.POINTER(ctypes.c_double), _i64p]),
 }

@@ -610,6 +610,84 @@ int msd_block_backward(int dtype, int ndim, int64_t batch, int64_t c_in, int dep
     return MSD_OK;
 }
 
+// ---------------------------------------------------------------------------
+// Final 1x1 layer (msd_module.py:60-88: Conv1d over the flattened voxels).
+// ---------------------------------------------------------------------------
+
+namespace {
+
+int check_final(const char *fn, int dtype, int64_t batch, int64_t c_in, int64_t c_out, int64_t nvox)
+{
+    if (dtype != MSD_F32 && dtype != MSD_F64) return fail(MSD_ERR_INVALID, "%s: dtype must be MSD_F32 or MSD_F64", fn);
+    if (batch <= 0 || c_in <= 0 || c_out <= 0 || nvox <= 0)
+        return fail(MSD_ERR_INVALID, "%s: batch, channel counts and voxel count must be positive", fn);
+    if (batch > 65535 || c_in > INT32_MAX || c_out > INT32_MAX)
+        return fail(MSD_ERR_INVALID, "%s: batch or channel count too large", fn);
+    return MSD_OK;
+}
+
+}  // namespace
+
+int64_t msd_final_workspace_bytes(int dtype, int64_t batch, int64_t c_in, int64_t c_out, int64_t nvox)
+{
+    if (check_final("msd_final_workspace_bytes", dtype, batch, c_in, c_out, nvox) != MSD_OK) return -1;
+    return msd::final_workspace_elems(batch, c_in, c_out, nvox) * (dtype == MSD_F32 ? 4 : 8);
+}
+
+int msd_final_forward(int dtype, int64_t batch, int64_t c_in, int64_t c_out, int64_t nvox, const void *input,
+                      int64_t input_batch_stride, int64_t input_channel_stride, const void *weight, const void *bias,
+                      void *output, int64_t output_batch_stride, int64_t output_channel_stride, void *stream)
+{
+    const char *fn = "final_forward";
+    MSD_TRY(check_final(fn, dtype, batch, c_in, c_out, nvox));
+    if (!input || !weight || !output) return fail(MSD_ERR_INVALID, "%s: NULL argument", fn);
+    if (input_batch_stride < 0 || input_channel_stride < 0 || output_batch_stride < 0 || output_channel_stride < 0)
+        return fail(MSD_ERR_INVALID, "%s: negative stride", fn);
+    const hipError_t e =
+        dtype == MSD_F32
+            ? msd::final_forward<float>(batch, (int)c_in, (int)c_out, nvox, (const float *)input, input_batch_stride,
+                                        input_channel_stride, (const float *)weight, (const float *)bias,
+                                        (float *)output, output_batch_stride, output_channel_stride,
+                                        (hipStream_t)stream)
+            : msd::final_forward<double>(batch, (int)c_in, (int)c_out, nvox, (const double *)input,
+                                         input_batch_stride, input_channel_stride, (const double *)weight,
+                                         (const double *)bias, (double *)output, output_batch_stride,
+                                         output_channel_stride, (hipStream_t)stream);
+    return e == hipSuccess ? MSD_OK : hip_fail(fn, e);
+}
+
+int msd_final_backward(int dtype, int64_t batch, int64_t c_in, int64_t c_out, int64_t nvox, const void *input,
+                       int64_t input_batch_stride, int64_t input_channel_stride, const void *grad_output,
+                       int64_t grad_output_batch_stride, int64_t grad_output_channel_stride, const void *weight,
+                       void *grad_input, int64_t grad_input_batch_stride, int64_t grad_input_channel_stride,
+                       void *grad_weight, void *grad_bias, void *workspace, int64_t workspace_bytes, void *stream)
+{
+    const char *fn = "final_backward";
+    MSD_TRY(check_final(fn, dtype, batch, c_in, c_out, nvox));
+    if (!input || !weight || !grad_output) return fail(MSD_ERR_INVALID, "%s: NULL argument", fn);
+    if (input_batch_stride < 0 || input_channel_stride < 0 || grad_output_batch_stride < 0 ||
+        grad_output_channel_stride < 0 || grad_input_batch_stride < 0 || grad_input_channel_stride < 0)
+        return fail(MSD_ERR_INVALID, "%s: negative stride", fn);
+    const int64_t need = msd_final_workspace_bytes(dtype, batch, c_in, c_out, nvox);
+    if (!workspace || workspace_bytes < need)
+        return fail(MSD_ERR_WORKSPACE, "%s: workspace of %lld bytes needed, %lld given", fn, (long long)need,
+                    (long long)(workspace ? workspace_bytes : 0));
+    const hipError_t e =
+        dtype == MSD_F32
+            ? msd::final_backward<float>(batch, (int)c_in, (int)c_out, nvox, (const float *)input, input_batch_stride,
+                                         input_channel_stride, (const float *)grad_output, grad_output_batch_stride,
+                                         grad_output_channel_stride, (const float *)weight, (float *)grad_input,
+                                         grad_input_batch_stride, grad_input_channel_stride, (float *)grad_weight,
+                                         (float *)grad_bias, (float *)workspace, (hipStream_t)stream)
+            : msd::final_backward<double>(batch, (int)c_in, (int)c_out, nvox, (const double *)input,
+                                          input_batch_stride, input_channel_stride, (const double *)grad_output,
+                                          grad_output_batch_stride, grad_output_channel_stride,
+                                          (const double *)weight, (double *)grad_input, grad_input_batch_stride,
+                                          grad_input_channel_stride, (double *)grad_weight, (double *)grad_bias,
+                                          (double *)workspace, (hipStream_t)stream);
+    return e == hipSuccess ? MSD_OK : hip_fail(fn, e);
+}
+
 int msd_profile_enable(int on)
 {
     g_profile.on = on != 0;

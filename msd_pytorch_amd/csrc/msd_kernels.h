@@ -34,6 +34,17 @@ template <typename T>
 hipError_t generic_backward_kb(const Geom &g, bool relu, View<const T> out, View<const T> gy, View<const T> x, T *gk,
                                T *gb, T *ws, hipStream_t s);
 
+// Final 1x1 layer over the channel stack (msd_final.hip); voxels are contiguous, batch and
+// channel strides in elements.  The backward overwrites gx, gw and gb (each may be null).
+int64_t final_workspace_elems(int64_t batch, int64_t c_in, int64_t c_out, int64_t nvox);
+template <typename T>
+hipError_t final_forward(int64_t batch, int c_in, int c_out, int64_t nvox, const T *x, int64_t xsb, int64_t xsc,
+                         const T *w, const T *bias, T *out, int64_t osb, int64_t osc, hipStream_t s);
+template <typename T>
+hipError_t final_backward(int64_t batch, int c_in, int c_out, int64_t nvox, const T *x, int64_t xsb, int64_t xsc,
+                          const T *go, int64_t gsb, int64_t gsc, const T *w, T *gx, int64_t gxsb, int64_t gxsc,
+                          T *gw, T *gb, T *ws, hipStream_t s);
+
 // Launch-shape knobs (msd_set_tuning in the C ABI).  A value < 0 means "library default".
 enum Knob {
     kKnobBwdxVec2d, kKnobBwdxVec3d, kKnobBwdxUnroll2d, kKnobBwdxUnroll3d, kKnobBwdxMinBlocks,

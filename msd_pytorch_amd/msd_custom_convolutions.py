@@ -387,3 +387,89 @@ def block_backward(stack, grads, c_in, dilations, weights, grad_weights, grad_bi
     _call("msd_block_backward", stack.device, *head, *_view(stack), *_view(grads), _ptr_array(weights),
           _ptr_array(grad_weights), ctypes.c_void_p(grad_bias.data_ptr() if grad_bias is not None else 0),
           1 if need_input_grad else 0, ctypes.c_void_p(ws.data_ptr()), int(need), _stream(stack))
+
+
+# ---------------------------------------------------------------------------
+# Final 1x1 layer over the channel stack (msd_module.py:60-88 of the reference,
+# which leaves it to torch's Conv1d).
+# ---------------------------------------------------------------------------
+
+def final_layer_supported(input):
+    """True when the native final layer can take ``input`` (B, C, *spatial) as it
+    is: on the GPU, float32/float64, every channel plane contiguous."""
+    if not input.is_cuda or input.dtype not in _DTYPES or input.dim() < 3:
+        return False
+    plane = input[0, 0]
+    return plane.is_contiguous() and input.numel() > 0
+
+
+def _flat_strides(t):
+    """(voxels per channel, batch stride, channel stride) of (B, C, *spatial)."""
+    nvox = 1
+    for s in t.shape[2:]:
+        nvox *= s
+    return nvox, t.stride(0), t.stride(1)
+
+
+def final_forward(input, weight, bias, output):
+    """output[b, o] = bias[o] + sum_c weight[o, c] * input[b, c]; weight is
+    (c_out, c_in) or Conv1d's (c_out, c_in, 1)."""
+    fn = "final_forward"
+    named = [("input", input), ("weight", weight), ("output", output)] + ([("bias", bias)] if bias is not None else [])
+    _check_same_gpu(fn, named)
+    _check_same_type(fn, named)
+    c_out, c_in = weight.shape[0], weight.shape[1]
+    if weight.numel() != c_out * c_in or not weight.is_contiguous():
+        _fail(fn, "Expected weight to be contiguous and shaped (c_out, c_in[, 1])")
+    if input.shape[1] != c_in or output.shape[1] != c_out or tuple(input.shape[2:]) != tuple(output.shape[2:]) \
+            or input.shape[0] != output.shape[0]:
+        _fail(fn, "Input shape does not match output shape. ")
+    if not (final_layer_supported(input) and final_layer_supported(output)):
+        _fail(fn, "Expected channel planes to be contiguous")
+    nvox, isb, isc = _flat_strides(input)
+    _, osb, osc = _flat_strides(output)
+    _call("msd_final_forward", input.device, _DTYPES[input.dtype], input.shape[0], c_in, c_out, nvox,
+          ctypes.c_void_p(input.data_ptr()), isb, isc, ctypes.c_void_p(weight.data_ptr()),
+          ctypes.c_void_p(bias.data_ptr() if bias is not None else 0), ctypes.c_void_p(output.data_ptr()), osb, osc,
+          _stream(input))
+
+
+def final_backward(input, grad_output, weight, grad_input, grad_weight, grad_bias):
+    """Gradients of final_forward; grad_input (or None), grad_weight (or None) and
+    grad_bias (or None) are OVERWRITTEN."""
+    fn = "final_backward"
+    named = [("input", input), ("grad_output", grad_output), ("weight", weight)]
+    named += [(n, t) for n, t in (("grad_input", grad_input), ("grad_weight", grad_weight), ("grad_bias", grad_bias))
+              if t is not None]
+    _check_same_gpu(fn, named)
+    _check_same_type(fn, named)
+    c_out, c_in = weight.shape[0], weight.shape[1]
+    if weight.numel() != c_out * c_in or not weight.is_contiguous():
+        _fail(fn, "Expected weight to be contiguous and shaped (c_out, c_in[, 1])")
+    if grad_weight is not None and (grad_weight.numel() != c_out * c_in or not grad_weight.is_contiguous()):
+        _fail(fn, "Expected grad_weight to be contiguous and shaped like weight")
+    if grad_bias is not None and (grad_bias.numel() != c_out or not grad_bias.is_contiguous()):
+        _fail(fn, "Expected grad_bias to be contiguous with c_out elements")
+    if input.shape[1] != c_in or grad_output.shape[1] != c_out or input.shape[0] != grad_output.shape[0] \
+            or tuple(input.shape[2:]) != tuple(grad_output.shape[2:]):
+        _fail(fn, "Input shape does not match output shape. ")
+    if grad_input is not None and tuple(grad_input.shape) != tuple(input.shape):
+        _fail(fn, "Input shape does not match output shape. ")
+    for t in (input, grad_output, grad_input):
+        if t is not None and not final_layer_supported(t):
+            _fail(fn, "Expected channel planes to be contiguous")
+    nvox, isb, isc = _flat_strides(input)
+    _, gsb, gsc = _flat_strides(grad_output)
+    xsb, xsc = (grad_input.stride(0), grad_input.stride(1)) if grad_input is not None else (0, 0)
+    lib = _native.load()
+    need = lib.msd_final_workspace_bytes(_DTYPES[input.dtype], input.shape[0], c_in, c_out, nvox)
+    if need < 0:
+        _fail(fn, _native.last_error())
+    ws = torch.empty(max(int(need), 8), dtype=torch.uint8, device=input.device)
+
+    def ptr(t):
+        return ctypes.c_void_p(t.data_ptr() if t is not None else 0)
+
+    _call("msd_final_backward", input.device, _DTYPES[input.dtype], input.shape[0], c_in, c_out, nvox, ptr(input), isb,
+          isc, ptr(grad_output), gsb, gsc, ptr(weight), ptr(grad_input), xsb, xsc, ptr(grad_weight), ptr(grad_bias),
+          ptr(ws), int(need), _stream(input))

@@ -3,6 +3,7 @@ from math import sqrt
 
 import torch
 
+from . import msd_custom_convolutions as cc
 from .msd_block import MSDBlock
 
 
@@ -22,11 +23,38 @@ def init_convolution_weights(conv_weight, c_in, c_out, width, depth):
     conv_weight.normal_(0, sqrt(2 / n))
 
 
+class MSDFinalFunction(torch.autograd.Function):
+    """out = bias + weight . stack over the channel axis, one native pass over the
+    stack forward and one backward (which produces the gradient of the whole stack)."""
+
+    @staticmethod
+    def forward(ctx, input, weight, bias):
+        ctx.save_for_backward(input, weight)
+        output = torch.empty(input.shape[0], weight.shape[0], *input.shape[2:], dtype=input.dtype,
+                             device=input.device)
+        cc.final_forward(input, weight, bias, output)
+        return output
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        input, weight = ctx.saved_tensors
+        if not cc.final_layer_supported(grad_output):
+            grad_output = grad_output.contiguous()
+        grad_input = torch.empty_like(input) if ctx.needs_input_grad[0] else None
+        grad_weight = torch.empty_like(weight) if ctx.needs_input_grad[1] else None
+        grad_bias = torch.empty(weight.shape[0], dtype=weight.dtype, device=weight.device) \
+            if ctx.needs_input_grad[2] else None
+        cc.final_backward(input, grad_output, weight, grad_input, grad_weight, grad_bias)
+        return grad_input, grad_weight, grad_bias
+
+
 class MSDFinalLayer(torch.nn.Module):
     """1x1 convolution over the whole channel stack, zero-initialised.
 
-    Stored as ``linear = Conv1d(c_in, c_out, 1)`` acting on a (B, C, voxels)
-    view, which keeps the state-dict keys of msd_module.py:60-88."""
+    The parameters live in ``linear = Conv1d(c_in, c_out, 1)``, which keeps the
+    state-dict keys of msd_module.py:60-88.  On the GPU the layer runs as one native
+    pass over the stack; elsewhere (CPU tensors, other dtypes) torch's Conv1d on the
+    (B, C, voxels) view computes it."""
 
     def __init__(self, c_in, c_out):
         super().__init__()
@@ -36,6 +64,8 @@ class MSDFinalLayer(torch.nn.Module):
         self.reset_parameters()
 
     def forward(self, input):
+        if cc.final_layer_supported(input) and input.dtype == self.linear.weight.dtype:
+            return MSDFinalFunction.apply(input, self.linear.weight, self.linear.bias)
         b, c, *size = input.shape
         flat = input.view(b, c, -1)
         return self.linear(flat).view(b, self.c_out, *size)

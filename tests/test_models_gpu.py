@@ -224,3 +224,51 @@ def test_segmentation_model_api(ndim, tmp_path):
     assert other.load(path) == 3
     assert abs(other.forward(x, labels) - model.forward(x, labels)) < 1e-6
     assert any(k.startswith("1.0.msd_block.weight") for k in model.net.state_dict())
+
+
+@pytest.mark.parametrize("shape,c_out,dtype", [
+    ((2, 7, 13, 21), 3, torch.float32),        # ragged voxel count: one voxel per thread
+    ((1, 101, 64, 64), 4, torch.float32),      # the stack of the headline network, 4 labels
+    ((2, 5, 6, 7, 8), 1, torch.float32),
+    ((1, 9, 8, 40), 11, torch.float32),        # more output channels than one launch takes (8 + 2 + 1)
+    ((2, 6, 9, 10), 2, torch.float64),
+    ((1, 3, 4, 6, 10), 5, torch.float64),
+])
+def test_final_layer_matches_conv1d(shape, c_out, dtype):
+    # the native final layer against the Conv1d over flattened voxels it replaces
+    # (reference msd_module.py:60-88), in double precision
+    from msd_pytorch_amd.msd_module import MSDFinalLayer
+    gen = torch.Generator().manual_seed(3)
+    b, c, *size = shape
+    # the layer's input is a channel slice of a larger stack in the network
+    stack = torch.randn(b, c + 2, *size, dtype=dtype, generator=gen).cuda()
+    x = stack[:, :c].detach().requires_grad_(True)
+    layer = MSDFinalLayer(c, c_out).to(dtype).cuda()
+    layer.linear.weight.data.copy_(torch.randn(c_out, c, 1, dtype=dtype, generator=gen))
+    layer.linear.bias.data.copy_(torch.randn(c_out, dtype=dtype, generator=gen))
+    g = torch.randn(b, c_out, *size, dtype=dtype, generator=gen).cuda()
+    out = layer(x)
+    out.backward(g)
+
+    xr = x.detach().double().requires_grad_(True)
+    wr = layer.linear.weight.detach().double().requires_grad_(True)
+    br = layer.linear.bias.detach().double().requires_grad_(True)
+    ref = torch.nn.functional.conv1d(xr.reshape(b, c, -1), wr, br).view(b, c_out, *size)
+    ref.backward(g.double())
+    tf, tg = (1e-5, 1e-4) if dtype == torch.float32 else (1e-12, 1e-11)
+    assert out.shape == ref.shape
+    assert rel_err(out, ref) <= tf
+    assert rel_err(x.grad, xr.grad) <= tg
+    assert rel_err(layer.linear.weight.grad, wr.grad) <= tg
+    assert rel_err(layer.linear.bias.grad, br.grad) <= tg
+
+
+def test_final_layer_without_input_gradient():
+    from msd_pytorch_amd.msd_module import MSDFinalLayer
+    layer = MSDFinalLayer(4, 2).cuda()
+    layer.linear.weight.data.normal_()
+    x = torch.randn(1, 4, 16, 16, device="cuda")
+    layer(x).sum().backward()
+    want = x.sum(dim=(0, 2, 3))
+    assert rel_err(layer.linear.weight.grad.view(2, 4)[0], want) <= 1e-4
+    assert abs(layer.linear.bias.grad[0].item() - 256.0) <= 1e-2
