@@ -208,7 +208,10 @@ inline bool make_lattice(const Geom &g, int V, int rz, int ry, int ks_wanted, La
     const int lpr = (need + kWave - 1) / kWave * kWave;
     if (lpr > 1024) return false;
     int ks = ks_wanted;
-    while (ks > 1 && (ks * lpr > 1024 || ks > g.C)) ks /= 2;
+    // 3D: at most 8 waves per workgroup, so that several workgroups share a CU and their
+    // phases (loads, arithmetic, LDS epilogue) overlap; long rows then split less
+    const int max_threads = g.ndim == 3 ? 512 : 1024;
+    while (ks > 1 && (ks * lpr > max_threads || ks > g.C)) ks /= 2;
     if ((size_t)ks * 3 * V * lpr * sizeof(float) > kMaxLds) return false;
     lt->lpr = lpr;
     lt->ks = ks;
