@@ -111,25 +111,28 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_rows_fused(const Args a, cons
 #pragma unroll
     for (int tg = 0; tg < TG; tg++) arow[tg] = min(tg * 16 + mj, K) * ASTRIDE + 4 * mk;
 
+    // Position of the lane's row, advanced from tile to tile without divisions: the row groups
+    // of a workgroup are consecutive.
+    int grp = lb * a.tiles_per_wg;
+    int gi = grp % a.ngroups, b = grp / a.ngroups;            // uniform: group within the image, batch index
+    int row = gi * rt.rpw + team;
+    int y = row % g.H, z = row / g.H;
+
     for (int ti = 0; ti < a.tiles_per_wg; ti++) {
-        const int grp = lb * a.tiles_per_wg + ti;
         if (grp >= a.total_groups) break;         // uniform over the workgroup
         int xsc = a.x.sc, gsc = a.gx.sc;
         asm volatile("" : "+s"(xsc), "+s"(gsc));  // keeps per-channel addresses from being hoisted out of the loop
-        const int b = grp / a.ngroups;
-        const int row = (grp % a.ngroups) * rt.rpw + team;
-        const bool rowok = row < rt.nrows;
+        const bool rowok = row < rt.nrows;        // teams past the last row work on it again and store nothing
         const bool act = rowok && x0 < g.W;
-        const int rr = min(row, rt.nrows - 1);
-        const int y = rr % g.H, z = rr / g.H;
+        const int zc = rowok ? z : g.D - 1, yc = rowok ? y : g.H - 1;
         // Addresses are a wave-uniform 64-bit base (scalar registers) plus a 32-bit byte offset
         // per lane, the form the memory instructions take directly.  x: the lane's channel is
         // part of the offset; grad_input and activations: the channel is part of the base.
         const uint64_t xbase = reinterpret_cast<uint64_t>(xp + (int64_t)b * a.x.sb);
-        const uint32_t xrow = (uint32_t)(z * a.x.sz + y * a.x.sy);
+        const uint32_t xrow = (uint32_t)(zc * a.x.sz + yc * a.x.sy);
         const uint64_t gbase = reinterpret_cast<uint64_t>(gxp + (int64_t)b * a.gx.sb);
         const uint64_t abase = reinterpret_cast<uint64_t>(actp + (int64_t)b * a.gx.sb);
-        uint32_t goff = 4u * (uint32_t)(z * a.gx.sz + y * a.gx.sy + xc);
+        uint32_t goff = 4u * (uint32_t)(zc * a.gx.sz + yc * a.gx.sy + xc);
         // uniform base of grad_input channel ci, kept in scalar registers
         auto channel_base = [&](uint64_t base, int ci) {
             uint64_t p = base + (uint64_t)((int64_t)ci * gsc * 4);
@@ -164,7 +167,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_rows_fused(const Args a, cons
             const View<const float> none{nullptr, 0, 0, 0, 0, 0};
             const View<const float> gyv{gyp, a.gy.sb, 0, a.gy.sz, a.gy.sy, 1};
             float own[1][NPQ][V];
-            stage_source_rows<NDIM, false, 1, V>(g, rt, none, gyv, b, z, y, lane, act, S, own);
+            stage_source_rows<NDIM, false, 1, V>(g, rt, none, gyv, b, zc, yc, lane, act, S, own);
             // per voxel: all LDS reads first, so that their latencies overlap, then the sums
 #pragma unroll
             for (int i = 0; i < V; i++) {
@@ -231,7 +234,8 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_rows_fused(const Args a, cons
         // `prefetch`: the weights of the next channel are requested right after the first use
         // of this channel's (scalar loads return in any order, so only a wait for all of them
         // exists: the request must follow that wait to have the rest of the arithmetic to land in)
-        auto update_channel = [&](int ci, float (&gv)[V], const float (&w)[K], auto prefetch, float (&wn)[K]) {
+        auto update_channel = [&](int ci, float (&gv)[V], const float (&w)[K], auto prefetch, float (&wn)[K],
+                                  bool masked) {
             float sum[V];
 #pragma unroll
             for (int i = 0; i < V; i++) sum[i] = w[0] * tv[0][i];
@@ -244,30 +248,39 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_rows_fused(const Args a, cons
                 for (int i = 0; i < V; i++) sum[i] += w[t] * tv[t][i];
 #pragma unroll
             for (int i = 0; i < V; i++) gv[i] += sum[i];
+            if (masked) {
+                // an output of the layer below: its gradient is complete with this update, so its
+                // ReLU mask is applied on the way out
+                float m[V];
+                load_global_vec<V>(channel_base(abase, ci), goff, m);
+#pragma unroll
+                for (int i = 0; i < V; i++) gv[i] = 0.f < m[i] ? gv[i] : 0.f;
+            }
             store_global_vec<V>(channel_base(gbase, ci), goff, gv);
         };
         // grad_input of one stage: up to NCS channels.  Lanes past the row sit the whole stage
-        // out, so that the channels form one straight run of code.
+        // out, so that the channels form one straight run of code; the stage that holds masked
+        // channels or the end of the channel range goes channel by channel instead.
         auto stage_x = [&](int cb, int h, float (&gg)[NCS][V]) {
             const int cj0 = c0 + cb * kChanBlock + h * NCS;
             if (!act) return;
             asm volatile("" : "+v"(goff));        // as in load_stage: the stores take base + lane offset directly
             float w[2][K];
-            if (cj0 + NCS <= cx_end) {            // uniform: all channels of the stage exist
+            if (cj0 + NCS <= min(cx_end, a.mask_from)) {   // uniform
                 load_weights(cj0, w[0]);
 #pragma unroll
                 for (int j = 0; j < NCS; j++) {
                     if (j + 1 < NCS)
-                        update_channel(cj0 + j, gg[j], w[j & 1], std::true_type{}, w[(j + 1) & 1]);
+                        update_channel(cj0 + j, gg[j], w[j & 1], std::true_type{}, w[(j + 1) & 1], false);
                     else
-                        update_channel(cj0 + j, gg[j], w[j & 1], std::false_type{}, w[(j + 1) & 1]);
+                        update_channel(cj0 + j, gg[j], w[j & 1], std::false_type{}, w[(j + 1) & 1], false);
                 }
             } else {
 #pragma unroll
                 for (int j = 0; j < NCS; j++)
                     if (cj0 + j < cx_end) {
                         load_weights(cj0 + j, w[0]);
-                        update_channel(cj0 + j, gg[j], w[0], std::false_type{}, w[1]);
+                        update_channel(cj0 + j, gg[j], w[0], std::false_type{}, w[1], cj0 + j >= a.mask_from);
                     }
             }
         };
@@ -294,21 +307,25 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_rows_fused(const Args a, cons
                     for (int tg = 0; tg < TG; tg++) D[q][tg] += acc[tg][0] + acc[tg][1];
                 }
         }
-        // Channels from mask_from on are outputs of the layer below: their gradient is complete
-        // with this update, so its ReLU mask is applied now (every lane revisits what it wrote).
-        if (act) {
-            for (int ci = max(a.mask_from, c0); ci < cx_end; ci++) {
-                float m[V], v[V];
-                load_global_vec<V>(channel_base(abase, ci), goff, m);
-                load_global_vec<V>(channel_base(gbase, ci), goff, v);
-#pragma unroll
-                for (int i = 0; i < V; i++) v[i] = 0.f < m[i] ? v[i] : 0.f;
-                store_global_vec<V>(channel_base(gbase, ci), goff, v);
-            }
-        }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        // next row group
+        grp++;
+        if (++gi == a.ngroups) {                  // uniform: first group of the next batch item
+            gi = 0;
+            b++;
+            row = team;
+            y = team % g.H;
+            z = team / g.H;
+        } else {
+            row += rt.rpw;
+            y += rt.rpw;
+            while (y >= g.H) {
+                y -= g.H;
+                z++;
+            }
+        }
     }
 
     // D[cb][tg][v] = sum for tap tg*16 + 4*mk + v, channel c0 + cb*16 + mj.  Add the waves in LDS.
