@@ -175,6 +175,24 @@ int msd_conv_backward_kb(int dtype, int ndim, int64_t batch, int64_t c_in, int64
                          void *grad_kernel, void *grad_bias,
                          void *workspace, int64_t workspace_bytes, void *stream);
 
+/* The three plain backward operators of one layer in one call:
+ *   grad_input += backward_x(grad_output, kernel), grad_kernel += backward_k(grad_output, input),
+ *   grad_bias += backward_bias(grad_output)   (grad_bias may be NULL)
+ * i.e. msd_block.py:107-126 for a grad_output that is already masked (msd_relu_mask_gradient).
+ * fp32 problems with one output channel, unit x-strides and rows of whole 4-voxel groups run
+ * as ONE pass over the input channels (the gather of grad_output is shared, input and
+ * grad_input are read once, grad_input written once); everything else runs the two
+ * operators one after the other.  grad_input must not alias input or grad_output.
+ * No counterpart in the reference. */
+int msd_conv_backward_xkb(int dtype, int ndim, int64_t batch, int64_t c_in, int64_t c_out,
+                          const int64_t *spatial, int dilation,
+                          const void *grad_output, const int64_t *grad_output_strides,
+                          const void *input, const int64_t *input_strides,
+                          const void *kernel,
+                          void *grad_input, const int64_t *grad_input_strides,
+                          void *grad_kernel, void *grad_bias,
+                          void *workspace, int64_t workspace_bytes, void *stream);
+
 /* grad_output = grad_output * [0 < output], in place: the ReLU mask that the three
  * conv_relu_backward_* operators of one layer (msd_block.py:107-126) each apply on
  * the fly, applied once.  After it the plain backward operators give the layer's

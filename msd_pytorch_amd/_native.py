@@ -39,6 +39,7 @@ PROTOTYPES = {
                                     + _WS + [_ptr]),
     "msd_conv_relu_backward_kb": (_c_int, _HEAD + _VIEW + _VIEW + _VIEW + [_ptr, _ptr] + _WS + [_ptr]),
     "msd_conv_backward_kb": (_c_int, _HEAD + _VIEW + _VIEW + [_ptr, _ptr] + _WS + [_ptr]),
+    "msd_conv_backward_xkb": (_c_int, _HEAD + _VIEW + _VIEW + [_ptr] + _VIEW + [_ptr, _ptr] + _WS + [_ptr]),
     "msd_relu_mask_gradient": (_c_int, [_c_int, _c_int, _c_i64, _c_i64, _i64p] + _VIEW + _VIEW + [_ptr]),
     "msd_block_workspace_bytes": (_c_i64, [_c_int, _c_int, _c_i64, _c_i64, _c_int, _i64p, _i64p]),
     "msd_block_forward": (_c_int, [_c_int, _c_int, _c_i64, _c_i64, _c_int, _i64p, _i64p, _i64p] + _VIEW

@@ -56,6 +56,9 @@ def bench_case(ndim, size, batch, c_in, width, dilation, iters, ops=("forward", 
                        (2 * c_in + 2 * width) * n * 4 + wbytes),
         "backward_kb": (lambda: cc.conv_relu_backward_kb(y, gy, x, gk, gb, dilation),
                         (c_in + 2 * width) * n * 4 + wbytes),
+        # the three plain backward operators in one call (what the dense block runs per layer)
+        "backward_xkb": (lambda: cc.conv_backward_xkb(gy, x, k, gx, gk, gb, dilation),
+                         (3 * c_in + 2 * width) * n * 4 + 2 * wbytes),
     }
     cc.conv_relu_forward(x, k, bias, y, dilation)
     rows = []

@@ -399,6 +399,42 @@ int msd_conv_backward_kb(int dtype, int ndim, int64_t batch, int64_t c_in, int64
                        workspace, workspace_bytes, stream);
 }
 
+int msd_conv_backward_xkb(int dtype, int ndim, int64_t batch, int64_t c_in, int64_t c_out, const int64_t *spatial,
+                          int dilation, const void *grad_output, const int64_t *grad_output_strides,
+                          const void *input, const int64_t *input_strides, const void *kernel, void *grad_input,
+                          const int64_t *grad_input_strides, void *grad_kernel, void *grad_bias, void *workspace,
+                          int64_t workspace_bytes, void *stream)
+{
+    const char *fn = "conv_backward_xkb";
+    if (!grad_kernel) return fail(MSD_ERR_INVALID, "%s: grad_kernel is NULL", fn);
+    if (dtype == MSD_F32 && g_kernel_path == 0 && ndim >= 2 && ndim <= 3) {
+        // one pass where the fused kernel covers the case
+        msd::Geom g;
+        MSD_TRY(make_geom(fn, dtype, ndim, batch, c_in, c_out, spatial, dilation, true, &g));
+        if (c_in <= 0) return fail(MSD_ERR_INVALID, "%s: c_in must be positive", fn);
+        if (!kernel) return fail(MSD_ERR_INVALID, "%s: kernel is NULL", fn);
+        msd::View<const float> gy, x;
+        msd::View<float> gx;
+        MSD_TRY(make_view(fn, "grad_output", ndim, grad_output, grad_output_strides, &gy));
+        MSD_TRY(make_view(fn, "input", ndim, input, input_strides, &x));
+        MSD_TRY(make_view(fn, "grad_input", ndim, grad_input, grad_input_strides, &gx));
+        if (msd::fast_backward_xkb_supported(g, gy, x, gx)) {
+            MSD_TRY(check_workspace(fn, g, sizeof(float), workspace, workspace_bytes));
+            const msd::PostMask none{g.C, {nullptr, 0, 0, 0, 0, 0}};
+            ProfileScope scope(3, (hipStream_t)stream);
+            const hipError_t e =
+                msd::fast_backward_xkb(g, gy, x, (const float *)kernel, gx, none, (float *)grad_kernel,
+                                       (float *)grad_bias, (float *)workspace, (hipStream_t)stream);
+            return e == hipSuccess ? MSD_OK : hip_fail(fn, e);
+        }
+    }
+    MSD_TRY(backward_x(fn, false, dtype, ndim, batch, c_in, c_out, spatial, dilation, nullptr, nullptr, grad_output,
+                       grad_output_strides, kernel, grad_input, grad_input_strides, stream));
+    return backward_kb(fn, false, true, dtype, ndim, batch, c_in, c_out, spatial, dilation, nullptr, nullptr,
+                       grad_output, grad_output_strides, input, input_strides, grad_kernel, grad_bias, workspace,
+                       workspace_bytes, stream);
+}
+
 int msd_relu_mask_gradient(int dtype, int ndim, int64_t batch, int64_t c_out, const int64_t *spatial,
                            const void *output, const int64_t *output_strides, void *grad_output,
                            const int64_t *grad_output_strides, void *stream)

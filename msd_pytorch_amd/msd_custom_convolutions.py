@@ -256,6 +256,42 @@ def conv_backward_kb(grad_output, input, grad_kernel, grad_bias, dilation, block
                 dilation, block_size)
 
 
+def conv_backward_xkb(grad_output, input, kernel, grad_input, grad_kernel, grad_bias, dilation, block_size=None):
+    """conv_backward_x, conv_backward_k and conv_backward_bias of one layer in one call
+    (one pass over the input channels where the fused kernel applies): grad_input,
+    grad_kernel and grad_bias (or None) are accumulated into.  Not part of the reference's
+    module."""
+    fn = "conv_backward_xkb"
+    named = [("grad_output", grad_output), ("input", input), ("kernel", kernel), ("grad_input", grad_input),
+             ("grad_kernel", grad_kernel)] + ([("grad_bias", grad_bias)] if grad_bias is not None else [])
+    _check_same_gpu(fn, named)
+    _check_same_type(fn, named)
+    _check_kernel(fn, kernel)
+    _check_kernel(fn, grad_kernel)
+    if tuple(kernel.shape) != tuple(grad_kernel.shape):
+        _fail(fn, "Expected grad_kernel to be shaped like kernel")
+    _check_in_out_shape(fn, input, grad_output)
+    if tuple(grad_input.shape) != tuple(input.shape):
+        _fail(fn, "Input shape does not match output shape. ")
+    for name, t in named[:5]:
+        _check_dim(fn, name, t, kernel.dim())
+    if kernel.shape[1] != input.shape[1]:
+        _fail(fn, "Kernel shape does not match input channels. ")
+    if kernel.shape[0] != grad_output.shape[1]:
+        _fail(fn, "Kernel shape does not match output channels. ")
+    if grad_bias is not None and (grad_bias.dim() != 1 or grad_bias.shape[0] != grad_output.shape[1]
+                                  or not grad_bias.is_contiguous()):
+        _fail(fn, "Bias shape does not match output channels. ")
+    _check_dilation(fn, input, dilation)
+    _check_block_size(fn, block_size)
+    c_in, c_out = input.shape[1], grad_output.shape[1]
+    ws, ws_ptr, ws_bytes = _workspace(input, c_in, c_out)
+    _call("msd_conv_backward_xkb", input.device, *_head(input, c_in, c_out, dilation), *_view(grad_output),
+          *_view(input), ctypes.c_void_p(kernel.data_ptr()), *_view(grad_input),
+          ctypes.c_void_p(grad_kernel.data_ptr()),
+          ctypes.c_void_p(grad_bias.data_ptr() if grad_bias is not None else 0), ws_ptr, ws_bytes, _stream(input))
+
+
 def relu_mask_gradient(output, grad_output):
     """grad_output *= (output > 0), in place: the mask the three conv_relu_backward_*
     operators of a layer apply on the fly, applied once (for callers that own

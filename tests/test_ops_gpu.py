@@ -162,3 +162,50 @@ def test_mask_once_then_plain_operators(cc, shape, dtype):
     cc.conv_backward_kb(gy, p["x"], gk1, gb1, p["d"])
     tol = 1e-5 if dtype == torch.float32 else 1e-12
     assert rel_err(gx1, gx0) <= tol and rel_err(gk1, gk0) <= tol and rel_err(gb1, gb0) <= tol
+
+
+# shapes the one-pass kernel behind conv_backward_xkb takes (one output channel, rows of whole
+# 4-voxel groups, at least one wavefront per row), beside the SHAPES_FAST ones that qualify
+SHAPES_XKB = [
+    (1, 17, 1, (5, 256), 2),          # 4 voxels per lane, 4 rows per workgroup, 2 channel blocks with the bias
+    (2, 3, 1, (9, 1024), 9),          # one row per workgroup, dilation == height
+    (1, 40, 1, (6, 7, 128), 3),       # 3D, 3 channel blocks
+    (1, 2, 1, (4, 5, 68), 4),         # 3D, ragged row
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("shape", SHAPES_XKB + [ALL_SHAPES[5], ALL_SHAPES[9], SHAPES_FAST[0], SHAPES_FAST[3],
+                                                SHAPES_FAST[5], SHAPES_FAST[6], SHAPES_FAST[9]])
+def test_backward_xkb_equals_the_three_operators(cc, shape, dtype):
+    # one call (one pass over the channels where the fused kernel applies; fp64, two output
+    # channels and odd row lengths take the separate kernels) against the oracle's
+    # conv_backward_x, conv_backward_k and conv_backward_bias, all accumulating
+    ref = make_problem(shape, dtype, seed=5)
+    dev = make_problem(shape, dtype, device="cuda", seed=5)
+    want_gk, want_gb = torch.ones_like(ref["k"]), torch.full_like(ref["bias"], 2.0)
+    oracle.conv_backward_x(ref["gy"], ref["k"], ref["gx"], ref["d"])
+    oracle.conv_backward_k(ref["gy"], ref["x"], want_gk, ref["d"])
+    oracle.conv_backward_bias(ref["gy"], want_gb)
+    got_gk, got_gb = torch.ones_like(dev["k"]), torch.full_like(dev["bias"], 2.0)
+    cc.conv_backward_xkb(dev["gy"], dev["x"], dev["k"], dev["gx"], got_gk, got_gb, dev["d"])
+    torch.cuda.synchronize()
+    assert rel_err(dev["gstack"], ref["gstack"]) <= TOL_GRAD[dtype], "grad_input"
+    assert torch.equal(dev["gy"].cpu(), ref["gy"]), "wrote outside grad_input"
+    assert rel_err(got_gk, want_gk) <= TOL_GRAD[dtype], "grad_kernel"
+    assert rel_err(got_gb, want_gb) <= TOL_GRAD[dtype], "grad_bias"
+
+
+def test_backward_xkb_without_bias_and_errors(cc):
+    p = make_problem(SHAPES_FAST[0], torch.float32, device="cuda")
+    gk = torch.zeros_like(p["k"])
+    gk2 = torch.zeros_like(p["k"])
+    gx2 = p["gx"].clone()
+    cc.conv_backward_xkb(p["gy"], p["x"], p["k"], p["gx"], gk, None, p["d"])
+    cc.conv_backward_x(p["gy"], p["k"], gx2, p["d"])
+    cc.conv_backward_k(p["gy"], p["x"], gk2, p["d"])
+    assert rel_err(p["gx"], gx2) <= 1e-5 and rel_err(gk, gk2) <= 1e-5
+    with pytest.raises(RuntimeError):
+        cc.conv_backward_xkb(p["gy"], p["x"], p["k"], p["gx"], gk, None, 65)      # dilation > size
+    with pytest.raises(RuntimeError):
+        cc.conv_backward_xkb(p["gy"].cpu(), p["x"], p["k"], p["gx"], gk, None, 1)  # CPU tensor
