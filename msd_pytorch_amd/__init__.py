@@ -8,6 +8,8 @@ from . import msd_custom_convolutions  # noqa: E402
 from . import conv2d, conv3d  # noqa: E402,F401
 from .msd_block import MSDBlock, MSDBlock2d, MSDBlock3d, MSDBlockFunction, msd_block  # noqa: E402,F401
 from .msd_module import MSDFinalLayer, MSDModule  # noqa: E402,F401
+from .errors import Error, InputError  # noqa: E402,F401
+from .image_dataset import ImageDataset, ImageStack  # noqa: E402,F401
 from .msd_regression_model import MSDRegressionModel  # noqa: E402,F401
 from .msd_segmentation_model import MSDSegmentationModel  # noqa: E402,F401
 

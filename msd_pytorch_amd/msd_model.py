@@ -33,16 +33,41 @@ def scaling_module_set_bias(sm, bias):
     sm.bias.data.fill_(bias)
 
 
-def _moments(batches):
-    """Mean and standard deviation from per-batch means of x and x**2."""
-    mean = square = 0
+def _moments(pairs):
+    """Mean and standard deviation of the inputs and of the targets of an iterable of
+    (input, target) batches, from per-batch means of x and x**2 as msd_model.py:140-153
+    computes them, in one pass and in double precision on the host."""
+    sums = [0.0, 0.0, 0.0, 0.0]
     n = 0
-    for x in batches:
-        mean = mean + x.mean()
-        square = square + x.pow(2).mean()
+    for pair in pairs:
+        x, y = pair[0], pair[1]
+        for i, t in enumerate((x, y)):
+            t = t.detach().double()
+            sums[2 * i] += float(t.mean())
+            sums[2 * i + 1] += float(t.pow(2).mean())
         n += 1
-    mean, square = mean / n, square / n
-    return float(mean), float(np.sqrt(float(square) - float(mean) ** 2))
+    if n == 0:
+        raise ValueError("set_normalization: the data loader yields no batches")
+    out = []
+    for i in range(2):
+        mean, square = sums[2 * i] / n, sums[2 * i + 1] / n
+        out += [mean, float(np.sqrt(max(square - mean ** 2, 0.0)))]
+    return tuple(out)
+
+
+def match_module_prefix(state_dict, wanted_keys):
+    """Rename the keys of a checkpoint so that it loads into a network with or without the
+    ``module.`` prefix that nn.DataParallel adds (``parallel=True`` models,
+    msd_regression_model.py:78-79): the prefix is added or dropped to agree with
+    ``wanted_keys``; a dictionary that already agrees is returned as it is."""
+    wanted = list(wanted_keys)
+    have_prefix = bool(state_dict) and all(k.startswith("module.") for k in state_dict)
+    want_prefix = bool(wanted) and all(k.startswith("module.") for k in wanted)
+    if have_prefix == want_prefix:
+        return state_dict
+    if have_prefix:
+        return type(state_dict)((k[len("module."):], v) for k, v in state_dict.items())
+    return type(state_dict)(("module." + k, v) for k, v in state_dict.items())
 
 
 class MSDModel:
@@ -70,8 +95,10 @@ class MSDModel:
     def set_normalization(self, dataloader):
         """Make scale_in map the training inputs to zero mean / unit variance
         and scale_out map the network output back to the targets' mean / std."""
-        mean_in, std_in = _moments(d[0] for d in dataloader)
-        mean_out, std_out = _moments(d[1] for d in dataloader)
+        mean_in, std_in, mean_out, std_out = _moments(dataloader)
+        if std_in == 0 or std_out == 0:
+            raise ValueError("set_normalization: the data has zero variance "
+                             f"(std of inputs {std_in}, of targets {std_out})")
         scaling_module_set_scale(self.scale_in, 1 / std_in)
         scaling_module_set_bias(self.scale_in, -mean_in / std_in)
         scaling_module_set_scale(self.scale_out, std_out)
@@ -136,9 +163,26 @@ class MSDModel:
         torch.save(state, path)
 
     def load(self, path):
-        """Restore network and optimiser; returns the stored epoch."""
-        state = torch.load(path, weights_only=True)
-        self.net.load_state_dict(state["state_dict"])
+        """Restore network and optimiser; returns the stored epoch.
+
+        Reads the files that ``save`` and the reference's ``save`` (msd_model.py:310-324)
+        write: ``{"epoch", "state_dict", "optimizer"}`` with the parameter names of the
+        reference (``weight{i}``, one flat ``bias``, ``final_layer.linear.*`` under the
+        position of the module in ``net``).  A checkpoint of a ``parallel=True`` model loads
+        into a plain one and the other way round.  Only tensors and plain containers are
+        accepted from the file (nothing in it is executed)."""
+        device = "cuda" if torch.cuda.is_available() else "cpu"
+        state = torch.load(path, map_location=device, weights_only=True)
+        missing = [k for k in ("epoch", "state_dict", "optimizer") if k not in state]
+        if missing:
+            raise RuntimeError(f"{path} is not an MSD checkpoint: no {missing} entry")
+        own = self.net.state_dict()
+        weights = match_module_prefix(state["state_dict"], own.keys())
+        for key, value in weights.items():
+            if key in own and tuple(own[key].shape) != tuple(value.shape):
+                raise RuntimeError(f"{path}: {key} has shape {tuple(value.shape)}, this model expects "
+                                   f"{tuple(own[key].shape)} (other depth, width or channel counts?)")
+        self.net.load_state_dict(weights)
         self.optimizer.load_state_dict(state["optimizer"])
         self.net.cuda()
         return state["epoch"]

@@ -21,7 +21,9 @@ class MSDSegmentationModel(MSDModel):
 
     def set_normalization(self, dataloader):
         """Only the input is normalised; the targets are labels."""
-        mean, std = _moments(d[0] for d in dataloader)
+        mean, std, _, _ = _moments(dataloader)
+        if std == 0:
+            raise ValueError("set_normalization: the input data has zero variance")
         scaling_module_set_scale(self.scale_in, 1 / std)
         scaling_module_set_bias(self.scale_in, -mean / std)
 

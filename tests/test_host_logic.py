@@ -250,13 +250,33 @@ def test_scaling_module_is_frozen_identity():
 
 def test_moments():
     torch.manual_seed(0)
-    batches = [torch.randn(4, 1, 8, 8) * 3 + 2 for _ in range(5)]
-    mean, std = _moments(batches)
-    allx = torch.cat(batches)
-    assert abs(mean - allx.mean().item()) < 1e-5
-    assert abs(std - allx.std(unbiased=False).item()) < 1e-4
+    pairs = [(torch.randn(4, 1, 8, 8) * 3 + 2, torch.randn(4, 2, 8, 8) * 0.5 - 1) for _ in range(5)]
+    mean_in, std_in, mean_out, std_out = _moments(iter(pairs))     # a one-shot iterable is enough
+    allx, ally = torch.cat([p[0] for p in pairs]), torch.cat([p[1] for p in pairs])
+    assert abs(mean_in - allx.mean().item()) < 1e-5
+    assert abs(std_in - allx.std(unbiased=False).item()) < 1e-4
+    assert abs(mean_out - ally.mean().item()) < 1e-5
+    assert abs(std_out - ally.std(unbiased=False).item()) < 1e-4
+    with pytest.raises(ValueError):
+        _moments([])
+
+
+def test_match_module_prefix():
+    from collections import OrderedDict
+    from msd_pytorch_amd.msd_model import match_module_prefix
+    plain = OrderedDict([("0.weight", 1), ("1.msd_block.weight0", 2), ("1.final_layer.linear.bias", 3)])
+    wrapped = OrderedDict(("module." + k, v) for k, v in plain.items())
+    assert match_module_prefix(plain, plain.keys()) is plain
+    assert match_module_prefix(wrapped, wrapped.keys()) is wrapped
+    stripped = match_module_prefix(wrapped, plain.keys())
+    assert list(stripped.items()) == list(plain.items()) and isinstance(stripped, OrderedDict)
+    assert list(match_module_prefix(plain, wrapped.keys()).items()) == list(wrapped.items())
+    # a dictionary where only some keys carry the prefix is left alone (load_state_dict reports it)
+    mixed = OrderedDict([("module.a", 1), ("b", 2)])
+    assert match_module_prefix(mixed, plain.keys()) is mixed
 
 
 def test_package_exports():
-    for name in ("MSDRegressionModel", "MSDSegmentationModel", "MSDModule", "MSDBlock2d", "MSDBlock3d"):
+    for name in ("MSDRegressionModel", "MSDSegmentationModel", "MSDModule", "MSDBlock2d", "MSDBlock3d",
+                 "ImageDataset", "ImageStack", "InputError"):
         assert hasattr(msd_pytorch_amd, name)

@@ -192,6 +192,65 @@ def test_regression_model_api(ndim, tmp_path):
         MSDRegressionModel(1, 1, 2, 1, ndim=4)
 
 
+def test_checkpoints_across_data_parallel_and_bad_files(tmp_path):
+    # a file in the layout the reference's save writes (msd_model.py:310-324), saved from a
+    # DataParallel net ("module." keys), loads into a plain model, and the other way round
+    from collections import OrderedDict
+    from msd_pytorch_amd import MSDRegressionModel
+    torch.manual_seed(1)
+    model = MSDRegressionModel(1, 1, depth=4, width=2, dilations=[1, 2])
+    x = torch.randn(2, 1, 16, 40)
+    y = x * 2 + 1
+    model.set_normalization([(x, y)])
+    for _ in range(3):
+        model.learn(x, y)
+    wrapped = OrderedDict(("module." + k, v.clone()) for k, v in model.net.state_dict().items())
+    path = os.path.join(tmp_path, "parallel.torch")
+    torch.save({"epoch": 11, "state_dict": wrapped, "optimizer": model.optimizer.state_dict()}, path)
+    other = MSDRegressionModel(1, 1, depth=4, width=2, dilations=[1, 2])
+    assert other.load(path) == 11
+    assert abs(other.forward(x, y) - model.forward(x, y)) < 1e-6
+    # the restored optimiser continues exactly like the original one
+    assert abs(other.learn(x, y) - model.learn(x, y)) < 1e-6
+    assert abs(other.forward(x, y) - model.forward(x, y)) < 1e-6
+    # plain file into a DataParallel model
+    plain = os.path.join(tmp_path, "plain.torch")
+    model.save(plain, 12)
+    par = MSDRegressionModel(1, 1, depth=4, width=2, dilations=[1, 2], parallel=True)
+    assert par.load(plain) == 12
+    assert all(k.startswith("module.") for k in par.net.state_dict())
+    assert abs(par.forward(x, y) - model.forward(x, y)) < 1e-6
+    # other architecture: a message that names the parameter
+    with pytest.raises(RuntimeError, match="msd_block.bias has shape"):
+        MSDRegressionModel(1, 1, depth=4, width=1, dilations=[1, 2]).load(plain)
+    with pytest.raises(RuntimeError):
+        MSDRegressionModel(1, 1, depth=5, width=2, dilations=[1, 2]).load(plain)
+    # not a checkpoint
+    bad = os.path.join(tmp_path, "bad.torch")
+    torch.save({"weights": 1}, bad)
+    with pytest.raises(RuntimeError, match="not an MSD checkpoint"):
+        model.load(bad)
+    with pytest.raises(ValueError, match="zero variance"):
+        model.set_normalization([(torch.ones(1, 1, 8, 8), y)])
+
+
+@pytest.mark.parametrize("task", ["regression", "segmentation"])
+def test_getting_started_example(task, tmp_path):
+    # the reference's examples/getting_started.py workflow on synthetic TIFF files:
+    # ImageDataset -> normalisation -> train -> save -> load -> predictions on disk
+    from msd_pytorch_amd.examples import getting_started
+    from msd_pytorch_amd.image_dataset import ImageStack
+    result = getting_started.main(["--task", task, "--epochs", "4", "--depth", "8", "--synthetic-size", "48",
+                                   "--synthetic-count", "6", "--labels", "0", "1", "2", "--out", str(tmp_path)])
+    train_errors = [h[0] for h in result["history"]]
+    assert all(e == e for e in train_errors) and train_errors[-1] < train_errors[0]
+    assert result["predictions"] == 3
+    outputs = ImageStack(tmp_path / "output_*.tif")
+    assert len(outputs) == 3 and outputs[0].shape == (1, 48, 48)
+    if task == "segmentation":
+        assert float(outputs[0].max()) <= 2
+
+
 def test_regression_state_dict_keys():
     # key layout of the reference's checkpoints (msd_regression_model.py:76, msd_block.py:170-179)
     from msd_pytorch_amd import MSDRegressionModel
