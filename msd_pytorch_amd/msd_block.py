@@ -14,24 +14,52 @@ import torch
 from . import msd_custom_convolutions as cc
 
 
+def block_stack_forward(input, dilations, bias, weights):
+    """The channel stack of the dense block: the input followed by every layer's output
+    (argument checks and layer loop of msd_block.py:8-58)."""
+    if len(dilations) != len(weights):
+        raise AssertionError("number of weights does not match depth")
+    if input.dim() not in (4, 5):
+        raise ValueError("Input to MSDBlock must be 2D or 3D")
+    widths = [w.shape[0] for w in weights]
+    if len(bias) != sum(widths):
+        raise AssertionError("number of biases does not match number of output channels from weights")
+    c_in = input.shape[1]
+    stack = input.new_empty(input.shape[0], c_in + sum(widths), *input.shape[2:])
+    stack[:, :c_in] = input
+    # the layer loop of msd_block.py:40-58 runs inside the native library
+    cc.block_forward(stack, c_in, list(dilations), bias, list(weights))
+    return stack
+
+
+def block_stack_backward(stack, grads, dilations, bias, weights, need_input, need_bias, need_weights):
+    """The reverse layer loop of msd_block.py:89-130 on ``grads``, the gradient of the
+    whole stack, which must be private to the caller: it is overwritten.  Returns
+    (grad_input, grad_bias, grad_weights).
+
+    Per layer the native library masks the layer's slice of ``grads`` once in place (the
+    slice is not read again afterwards) and then applies the plain backward operators;
+    the reference masks on the fly in each of conv_relu_backward_x / _k / _bias."""
+    grad_bias = torch.zeros_like(bias) if need_bias else None
+    grad_weights = [None] * len(weights)
+    # one zero-filled buffer for all weight gradients (one fill instead of one per layer)
+    wanted = [w for w, need in zip(weights, need_weights) if need]
+    flat = stack.new_zeros(sum(w.numel() for w in wanted))
+    offset = 0
+    for idx, weight in enumerate(weights):
+        if need_weights[idx]:
+            grad_weights[idx] = flat[offset:offset + weight.numel()].view_as(weight)
+            offset += weight.numel()
+    c_in = weights[0].shape[1]
+    cc.block_backward(stack, grads, c_in, list(dilations), list(weights), grad_weights,
+                      grad_bias if need_bias else None, bool(need_input))
+    return (grads[:, :c_in] if need_input else None), grad_bias, grad_weights
+
+
 class MSDBlockFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, input, dilations, bias, *weights):
-        if len(dilations) != len(weights):
-            raise AssertionError("number of weights does not match depth")
-        if input.dim() not in (4, 5):
-            raise ValueError("Input to MSDBlock must be 2D or 3D")
-        widths = [w.shape[0] for w in weights]
-        if len(bias) != sum(widths):
-            raise AssertionError("number of biases does not match number of output channels from weights")
-
-        c_in = input.shape[1]
-        stack = input.new_empty(input.shape[0], c_in + sum(widths), *input.shape[2:])
-        stack[:, :c_in] = input
-
-        # the layer loop of msd_block.py:40-58 runs inside the native library
-        cc.block_forward(stack, c_in, list(dilations), bias, list(weights))
-
+        stack = block_stack_forward(input, dilations, bias, weights)
         ctx.dilations = tuple(dilations)
         ctx.save_for_backward(bias, stack, *weights)
         return stack
@@ -42,30 +70,12 @@ class MSDBlockFunction(torch.autograd.Function):
         if grad_output.dim() != stack.dim():
             raise AssertionError("Mismatched tensor dimensions.")
         need_input, _, need_bias, *need_weights = ctx.needs_input_grad
-
-        # Working copy of the incoming gradient: layer idx adds its input
-        # gradient to channels [0, first), which later iterations consume.
+        # Working copy of the incoming gradient (autograd may hand the same tensor to
+        # others): layer idx adds its input gradient to channels [0, first), which later
+        # iterations consume.
         grads = grad_output.clone()
-        grad_bias = torch.zeros_like(bias) if need_bias else None
-        grad_weights = [None] * len(weights)
-
-        # The reverse layer loop of msd_block.py:89-130 runs inside the native library.
-        # Per layer it masks the layer's slice of `grads` once in place (the slice is
-        # private to this call and not read again afterwards) and then applies the
-        # plain backward operators; the reference masks on the fly in each of
-        # conv_relu_backward_x / _k / _bias.
-        # one zero-filled buffer for all weight gradients (one fill instead of one per layer)
-        wanted = [w for w, need in zip(weights, need_weights) if need]
-        flat = stack.new_zeros(sum(w.numel() for w in wanted))
-        offset = 0
-        for idx, weight in enumerate(weights):
-            if need_weights[idx]:
-                grad_weights[idx] = flat[offset:offset + weight.numel()].view_as(weight)
-                offset += weight.numel()
-        cc.block_backward(stack, grads, weights[0].shape[1], list(ctx.dilations), list(weights), grad_weights,
-                          grad_bias if need_bias else None, bool(need_input))
-
-        grad_input = grads[:, :weights[0].shape[1]] if need_input else None
+        grad_input, grad_bias, grad_weights = block_stack_backward(
+            stack, grads, ctx.dilations, bias, weights, need_input, need_bias, need_weights)
         return (grad_input, None, grad_bias, *grad_weights)
 
 

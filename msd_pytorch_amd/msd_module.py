@@ -4,7 +4,7 @@ from math import sqrt
 import torch
 
 from . import msd_custom_convolutions as cc
-from .msd_block import MSDBlock
+from .msd_block import MSDBlock, block_stack_backward, block_stack_forward
 
 
 def units_in_front(c_in, width, layer_depth):
@@ -46,6 +46,45 @@ class MSDFinalFunction(torch.autograd.Function):
             if ctx.needs_input_grad[2] else None
         cc.final_backward(input, grad_output, weight, grad_input, grad_weight, grad_bias)
         return grad_input, grad_weight, grad_bias
+
+
+class MSDNetFunction(torch.autograd.Function):
+    """Dense block and final layer as ONE autograd node:
+    ``(input, dilations, bias, final_weight, final_bias, *weights) -> output``.
+
+    Same values as ``MSDFinalFunction(MSDBlockFunction(...))``.  The channel stack stays
+    inside the node, so in backward the final layer writes the gradient of the whole stack
+    straight into a fresh buffer that the block's reverse loop then owns: the stack-sized
+    copy that MSDBlockFunction.backward has to take of its incoming gradient
+    (msd_block.py:82-83) is not needed."""
+
+    @staticmethod
+    def forward(ctx, input, dilations, bias, final_weight, final_bias, *weights):
+        stack = block_stack_forward(input, dilations, bias, weights)
+        output = torch.empty(input.shape[0], final_weight.shape[0], *input.shape[2:], dtype=input.dtype,
+                             device=input.device)
+        cc.final_forward(stack, final_weight, final_bias, output)
+        ctx.dilations = tuple(dilations)
+        ctx.save_for_backward(bias, stack, final_weight, *weights)
+        return output
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        bias, stack, final_weight, *weights = ctx.saved_tensors
+        need_input, _, need_bias, need_fw, need_fb, *need_weights = ctx.needs_input_grad
+        if not cc.final_layer_supported(grad_output):
+            grad_output = grad_output.contiguous()
+        block_needed = need_input or need_bias or any(need_weights)
+        grads = torch.empty_like(stack) if block_needed else None
+        grad_fw = torch.empty_like(final_weight) if need_fw else None
+        grad_fb = torch.empty(final_weight.shape[0], dtype=final_weight.dtype, device=final_weight.device) \
+            if need_fb else None
+        cc.final_backward(stack, grad_output, final_weight, grads, grad_fw, grad_fb)
+        grad_input, grad_bias, grad_weights = (None, None, [None] * len(weights))
+        if block_needed:
+            grad_input, grad_bias, grad_weights = block_stack_backward(
+                stack, grads, ctx.dilations, bias, weights, need_input, need_bias, need_weights)
+        return (grad_input, None, grad_bias, grad_fw, grad_fb, *grad_weights)
 
 
 class MSDFinalLayer(torch.nn.Module):
@@ -107,5 +146,20 @@ class MSDModule(torch.nn.Module):
         self.msd_block.bias.data.zero_()
         self.final_layer.reset_parameters()
 
+    def _hooked(self):
+        """True when a hook sits on the block, the final layer or its Conv1d: hooks see
+        the modules' own calls, so the modules are then called one by one."""
+        for m in (self.msd_block, self.final_layer, self.final_layer.linear):
+            if m._forward_hooks or m._forward_pre_hooks or m._backward_hooks or m._backward_pre_hooks:
+                return True
+        return False
+
     def forward(self, input):
+        linear = self.final_layer.linear
+        if cc.final_layer_supported(input) and input.dim() in (4, 5) and input.dtype == linear.weight.dtype \
+                and linear.bias is not None and not self._hooked():
+            # block + final layer as one autograd node (no copy of the stack's gradient)
+            block = self.msd_block
+            weights = (getattr(block, f"weight{i}") for i in range(len(block.weights)))
+            return MSDNetFunction.apply(input, block.dilations, block.bias, linear.weight, linear.bias, *weights)
         return self.final_layer(self.msd_block(input))

@@ -160,6 +160,55 @@ def test_module_zero_output_then_all_parameters_move():
         assert not torch.equal(b, p.detach())
 
 
+@pytest.mark.parametrize("ndim,size,dtype", [(2, (33, 70), torch.float32), (3, (9, 12, 40), torch.float32),
+                                             (2, (12, 17), torch.float64)])
+def test_module_as_one_node_equals_block_then_final_layer(ndim, size, dtype):
+    # MSDModule.forward runs block + final layer as one autograd node; the two modules called
+    # one after the other (the reference's msd_module.py:144-146) must give the same bits
+    from msd_pytorch_amd import MSDModule
+    torch.manual_seed(3)
+    net = MSDModule(2, 3, depth=6, width=2, dilations=[1, 2, 3], ndim=ndim).cuda().to(dtype)
+    net.final_layer.linear.weight.data.normal_(0, 0.3)
+    net.final_layer.linear.bias.data.normal_(0, 0.3)
+    x = torch.randn(2, 2, *size, device="cuda", dtype=dtype, requires_grad=True)
+    g = torch.randn(2, 3, *size, device="cuda", dtype=dtype)
+
+    def run(forward):
+        for p in net.parameters():
+            p.grad = None
+        x.grad = None
+        out = forward(x)
+        out.backward(g)
+        return [out.detach().clone(), x.grad.clone()] + [p.grad.clone() for p in net.parameters()]
+
+    one = run(net)
+    two = run(lambda t: net.final_layer(net.msd_block(t)))
+    assert len(one) == len(two) == 2 + len(list(net.parameters()))
+    for a, b in zip(one, two):
+        assert torch.equal(a, b)
+    # a hook on a sub-module is honoured: the modules are then called one by one
+    seen = []
+    handle = net.msd_block.register_forward_hook(lambda m, i, o: seen.append(tuple(o.shape)))
+    hooked = run(net)
+    handle.remove()
+    assert seen == [(2, 2 + 6 * 2, *size)]
+    for a, b in zip(one, hooked):
+        assert torch.equal(a, b)
+    # gradients only for the final layer, or only for the input
+    for p in net.msd_block.parameters():
+        p.requires_grad_(False)
+    out = net(x.detach())
+    out.backward(g)
+    assert net.final_layer.linear.weight.grad is not None
+    for p in net.parameters():
+        p.requires_grad_(False)
+    x.grad = None
+    net(x).backward(g)
+    assert torch.equal(x.grad, one[1])
+    with torch.no_grad():
+        assert torch.equal(net(x), one[0])
+
+
 @pytest.mark.parametrize("ndim", [2, 3])
 def test_regression_model_api(ndim, tmp_path):
     # reference tests/test_msd_regression_model.py:8-143
