@@ -216,7 +216,11 @@ int msd_relu_mask_gradient(int dtype, int ndim, int64_t batch, int64_t c_out, co
  * is the private working copy of msd_block.py:83); on return channels [0, c_in) hold
  * dL/dinput (if need_input_grad).  grad_weights[i] (zero-filled by the caller, NULL to
  * skip a layer) and grad_bias (zero-filled, NULL to skip) are accumulated into.
- * Replaces the loop of msd_block.py:89-130.  Workspace: msd_block_workspace_bytes.
+ * Replaces the loop of msd_block.py:89-130.  Workspace: msd_block_workspace_bytes,
+ * which is the largest msd_workspace_bytes of the layers plus room (at most 1 GiB) for
+ * the partial weight-gradient sums of many layers at once, so that one launch can
+ * reduce up to 16 layers; the largest msd_workspace_bytes of the layers alone is
+ * accepted too (every layer then reduces its sums right away; same results).
  */
 int64_t msd_block_workspace_bytes(int dtype, int ndim, int64_t batch, int64_t c_in, int depth,
                                   const int64_t *widths, const int64_t *spatial);

@@ -15,8 +15,9 @@ const char *const kKnobNames[kKnobCount] = {
     "bwdx.vec2d", "bwdx.vec3d", "bwdx.unroll2d", "bwdx.unroll3d", "bwdx.min_blocks",
     "xcd_remap", "bwdk.vec2d", "bwdk.vec3d", "bwdk.blocks",
     "fwd.vec2d", "fwd.vec3d", "fwd.split", "fwd.rows2d", "bwdk.rows", "block.fuse",
+    "block.defer",
 };
-int g_knobs[kKnobCount] = {-1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1};
+int g_knobs[kKnobCount] = {-1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1};
 int knob(Knob k, int dflt) { return g_knobs[k] < 0 ? dflt : g_knobs[k]; }
 }  // namespace msd
 
@@ -38,7 +39,11 @@ struct Profile {
     bool on = false;
     std::vector<hipEvent_t> pool;                           // reused across calls
     size_t used = 0;
-    std::vector<std::pair<size_t, size_t>> spans[kProfileClasses];        // (start, stop) indices into pool
+    struct Span {
+        size_t start, stop;                                  // indices into pool
+        bool counted;                                        // adds to the class's number of calls
+    };
+    std::vector<Span> spans[kProfileClasses];
     hipEvent_t take()
     {
         if (used == pool.size()) {
@@ -50,13 +55,16 @@ struct Profile {
     }
 } g_profile;
 
-// Records an event pair around the launches made during its lifetime.
+// Records an event pair around the launches made during its lifetime.  `counted` false:
+// the time is added to the class, the number of calls is not (work done on behalf of calls
+// that were counted already).
 struct ProfileScope {
     int cls;
     hipStream_t s;
     size_t start = 0;
-    bool active;
-    ProfileScope(int cls_, hipStream_t s_) : cls(cls_), s(s_), active(g_profile.on)
+    bool active, counted;
+    ProfileScope(int cls_, hipStream_t s_, bool counted_ = true)
+        : cls(cls_), s(s_), active(g_profile.on), counted(counted_)
     {
         if (!active) return;
         start = g_profile.used;
@@ -68,7 +76,7 @@ struct ProfileScope {
         if (!active) return;
         const size_t stop = g_profile.used;
         hipEvent_t e = g_profile.take();
-        if (e && hipEventRecord(e, s) == hipSuccess) g_profile.spans[cls].push_back({start, stop});
+        if (e && hipEventRecord(e, s) == hipSuccess) g_profile.spans[cls].push_back({start, stop, counted});
     }
 };
 
@@ -514,10 +522,71 @@ int check_block(const char *fn, int dtype, int ndim, int64_t batch, int64_t c_in
 // [0, first) += backward_x, grad_weights/grad_bias += backward_k/bias, the ReLU mask of the
 // layer below applied to its channels on the way out.  *done is false (and nothing was
 // launched) when the fused kernel does not cover the case.
+// Floats of workspace that the partial sums of one fused layer take (one output channel).
+int64_t partial_region_floats(int ndim, int64_t c_in)
+{
+    return (c_in * (ndim == 3 ? 27 : 9) + 1) * (int64_t)msd::kMaxPartialRows;
+}
+
+constexpr int64_t kDeferBudgetBytes = (int64_t)1 << 30;   // most workspace spent on pending partial sums
+
+// Largest workspace a single layer of the block asks for, rounded up to 256 bytes: the
+// regions of the pending reductions start there.
+int64_t block_layer_workspace(int dtype, int ndim, int64_t batch, int64_t c_in, int depth, const int64_t *widths,
+                              const int64_t *spatial)
+{
+    int64_t total = c_in, need = 0;
+    for (int i = 0; i < depth; i++) {
+        if (widths[i] <= 0) return -1;
+        const int64_t n = msd_workspace_bytes(dtype, ndim, batch, total, widths[i], spatial);
+        if (n < 0) return -1;
+        need = n > need ? n : need;
+        total += widths[i];
+    }
+    return (need + 255) / 256 * 256;
+}
+
+// The reverse loop's pending column reductions: each fused layer leaves its partial sums in
+// a region of its own behind the per-layer workspace, and one launch reduces up to
+// kReduceBatch layers (a reduction per layer is a 4 microsecond launch between two large
+// kernels).  With no room for regions every layer reduces at once, as the single operators do.
+struct DeferredReductions {
+    float *base = nullptr;
+    int64_t capacity = 0, cursor = 0;             // floats
+    msd::ReduceJob jobs[msd::kReduceBatch];
+    int n = 0;
+    hipStream_t s = nullptr;
+
+    int flush(const char *fn)
+    {
+        if (n == 0) return MSD_OK;
+        ProfileScope scope(3, s, false);
+        const hipError_t e = msd::reduce_columns_batch(jobs, n, s);
+        n = 0;
+        cursor = 0;
+        return e == hipSuccess ? MSD_OK : hip_fail(fn, e);
+    }
+    // the job to hand to the next fused layer, its region set; nullptr when the region cannot fit
+    int next(const char *fn, int64_t floats, msd::ReduceJob **job)
+    {
+        *job = nullptr;
+        if (!base || floats > capacity) return MSD_OK;
+        if (n == msd::kReduceBatch || cursor + floats > capacity) MSD_TRY(flush(fn));
+        jobs[n].part = base + cursor;
+        *job = &jobs[n];
+        return MSD_OK;
+    }
+    void taken(int64_t floats)
+    {
+        n++;
+        cursor += floats;
+    }
+};
+
 int block_layer_fused(const char *fn, const BlockArgs &a, int i, int64_t first, const void *stack,
                       const int64_t *stack_strides, void *grads, const int64_t *grads_strides, const void *gout_i,
                       const void *weights_i, void *gk, void *gb, void *ws, int64_t ws_bytes, hipStream_t s,
-                      bool *masked, bool *done)
+                      DeferredReductions *pending, bool *masked, bool *done)
 {
     *done = false;
     if (a.dtype != MSD_F32 || g_kernel_path != 0 || !gk || !msd::knob(msd::kKnobBlockFuse, 1)) return MSD_OK;
@@ -541,10 +610,14 @@ int block_layer_fused(const char *fn, const BlockArgs &a, int i, int64_t first, 
             *masked = true;
         }
     }
+    const int64_t region = partial_region_floats(a.ndim, g.C);
+    msd::ReduceJob *job = nullptr;
+    MSD_TRY(pending->next(fn, region, &job));
     ProfileScope scope(3, s);
     const hipError_t e = msd::fast_backward_xkb(g, gy, x, (const float *)weights_i, gx, pm, (float *)gk, (float *)gb,
-                                                (float *)ws, s);
+                                                (float *)ws, s, job);
     if (e != hipSuccess) return hip_fail(fn, e);
+    if (job) pending->taken(region);
     *done = true;
     return MSD_OK;
 }
@@ -555,16 +628,16 @@ int64_t msd_block_workspace_bytes(int dtype, int ndim, int64_t batch, int64_t c_
                                   const int64_t *spatial)
 {
     if (!widths || depth <= 0) return -1;
-    int64_t total = c_in, wmax = 0, need = 0;
+    const int64_t need = block_layer_workspace(dtype, ndim, batch, c_in, depth, widths, spatial);
+    if (need < 0) return -1;
+    // behind it: regions for the partial sums of the layers the fused kernel can take, so that
+    // their reductions can wait for one another
+    int64_t regions = 0, total = c_in;
     for (int i = 0; i < depth; i++) {
-        if (widths[i] <= 0) return -1;
-        wmax = widths[i] > wmax ? widths[i] : wmax;
-        const int64_t n = msd_workspace_bytes(dtype, ndim, batch, total, widths[i], spatial);
-        if (n < 0) return -1;
-        need = n > need ? n : need;
+        if (dtype == MSD_F32 && widths[i] == 1) regions += partial_region_floats(ndim, total) * (int64_t)sizeof(float);
         total += widths[i];
     }
-    return need;
+    return need + (regions < kDeferBudgetBytes ? regions : kDeferBudgetBytes);
 }
 
 int msd_block_forward(int dtype, int ndim, int64_t batch, int64_t c_in, int depth, const int64_t *widths,
@@ -600,6 +673,13 @@ int msd_block_backward(int dtype, int ndim, int64_t batch, int64_t c_in, int dep
                         weights, &a));
     if (!grads || !grads_strides || !grad_weights) return fail(MSD_ERR_INVALID, "%s: NULL argument", fn);
     int64_t last = a.c_total, b1 = a.c_total - c_in;
+    DeferredReductions pending;
+    pending.s = (hipStream_t)stream;
+    const int64_t layer_ws = block_layer_workspace(dtype, ndim, batch, c_in, depth, widths, spatial);
+    if (workspace && layer_ws >= 0 && workspace_bytes > layer_ws && msd::knob(msd::kKnobBlockDefer, 1)) {
+        pending.base = (float *)((char *)workspace + layer_ws);
+        pending.capacity = (workspace_bytes - layer_ws) / (int64_t)sizeof(float);
+    }
     bool masked = false;   // the mask of the current layer was already applied by the previous backward_x
     for (int i = depth - 1; i >= 0; i--) {
         const int64_t w = widths[i], first = last - w, b0 = b1 - w;
@@ -619,8 +699,8 @@ int msd_block_backward(int dtype, int ndim, int64_t batch, int64_t c_in, int dep
             // one pass for the input, weight and bias gradients where the fused kernel applies
             bool done = false;
             MSD_TRY(block_layer_fused(fn, a, i, first, stack, stack_strides, grads, grads_strides, gout_i, weights[i],
-                                      grad_weights[i], gb, workspace, workspace_bytes, (hipStream_t)stream, &masked,
-                                      &done));
+                                      grad_weights[i], gb, workspace, workspace_bytes, (hipStream_t)stream, &pending,
+                                      &masked, &done));
             if (done) {
                 last = first;
                 b1 = b0;
@@ -643,7 +723,7 @@ int msd_block_backward(int dtype, int ndim, int64_t batch, int64_t c_in, int dep
         last = first;
         b1 = b0;
     }
-    return MSD_OK;
+    return pending.flush(fn);
 }
 
 // ---------------------------------------------------------------------------
@@ -737,15 +817,17 @@ int msd_profile_read(double *ms, int64_t *calls)
     if (!ms || !calls) return fail(MSD_ERR_INVALID, "msd_profile_read: NULL argument");
     for (int c = 0; c < kProfileClasses; c++) {
         double total = 0;
+        int64_t ncalls = 0;
         for (const auto &sp : g_profile.spans[c]) {
-            hipError_t e = hipEventSynchronize(g_profile.pool[sp.second]);
+            hipError_t e = hipEventSynchronize(g_profile.pool[sp.stop]);
             float t = 0;
-            if (e == hipSuccess) e = hipEventElapsedTime(&t, g_profile.pool[sp.first], g_profile.pool[sp.second]);
+            if (e == hipSuccess) e = hipEventElapsedTime(&t, g_profile.pool[sp.start], g_profile.pool[sp.stop]);
             if (e != hipSuccess) return hip_fail("msd_profile_read", e);
             total += t;
+            ncalls += sp.counted ? 1 : 0;
         }
         ms[c] = total;
-        calls[c] = (int64_t)g_profile.spans[c].size();
+        calls[c] = ncalls;
     }
     return MSD_OK;
 }

@@ -11,9 +11,9 @@ bool fast_backward_xkb_supported_2d(const Geom &g, const View<const float> &gy, 
 
 hipError_t fast_backward_xkb_2d(const Geom &g, const View<const float> &gy, const View<const float> &x, const float *k,
                                 const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws,
-                                hipStream_t s)
+                                hipStream_t s, ReduceJob *defer)
 {
-    return bwdxk::xkb_nd<2>(g, gy, x, k, gx, pm, gk, gb, ws, s);
+    return bwdxk::xkb_nd<2>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
 }
 
 }  // namespace msd

@@ -399,13 +399,15 @@ int choose_vec(const Geom &g, int vmax, const View<const float> &gy, const View<
 
 template <int NDIM, int V, int NCB>
 hipError_t launch(const Geom &g, const View<const float> &gy, const View<const float> &x, const float *k,
-                  const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws, hipStream_t s)
+                  const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws, hipStream_t s,
+                  ReduceJob *defer)
 {
     constexpr int K = Taps<NDIM>::K;
     Args a;
     a.g = g;
     make_row_teams(g, V, &a.rt);
-    float *part = ws + backward_k_mask_floats(g);
+    // a deferred reduction brings its own region for the partial sums (defer->part)
+    float *part = defer ? const_cast<float *>(defer->part) : ws + backward_k_mask_floats(g);
     a.ngroups = (a.rt.nrows + a.rt.rpw - 1) / a.rt.rpw;
     const int64_t total = (int64_t)a.ngroups * g.B;
     a.remap = knob(kKnobXcdRemap, 1);
@@ -430,19 +432,24 @@ hipError_t launch(const Geom &g, const View<const float> &gy, const View<const f
     if (e != hipSuccess) return e;
     const int64_t nk = (int64_t)g.C * K;
     const int64_t ncols = nk + (a.want_bias ? 1 : 0);
+    if (defer) {
+        *defer = ReduceJob{part, gk, gb, nk, ncols, rows};
+        return hipSuccess;
+    }
     hipLaunchKernelGGL(bwdk::reduce_columns, dim3((ncols + 3) / 4), dim3(256), 0, s, part, rows, nk, ncols, gk, gb);
     return hipGetLastError();
 }
 
 template <int NDIM, int V>
 hipError_t pick_ncb(const Geom &g, const View<const float> &gy, const View<const float> &x, const float *k,
-                    const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws, hipStream_t s)
+                    const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws, hipStream_t s,
+                    ReduceJob *defer)
 {
     const int need = (g.C + (gb != nullptr) + kChanBlock - 1) / kChanBlock;
-    if (need <= 1) return launch<NDIM, V, 1>(g, gy, x, k, gx, pm, gk, gb, ws, s);
-    if (need <= 2) return launch<NDIM, V, 2>(g, gy, x, k, gx, pm, gk, gb, ws, s);
-    if (need <= 4) return launch<NDIM, V, 4>(g, gy, x, k, gx, pm, gk, gb, ws, s);
-    return launch<NDIM, V, 8>(g, gy, x, k, gx, pm, gk, gb, ws, s);
+    if (need <= 1) return launch<NDIM, V, 1>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
+    if (need <= 2) return launch<NDIM, V, 2>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
+    if (need <= 4) return launch<NDIM, V, 4>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
+    return launch<NDIM, V, 8>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
 }
 
 // One output channel, unit x-strides, 32-bit strides, and a vector width that fits.
@@ -458,17 +465,18 @@ bool xkb_supported_nd(const Geom &g, const View<const float> &gy, const View<con
 // pm.act, where pm.from < C, must be laid out like gx (same strides and 16-byte phase).
 template <int NDIM>
 hipError_t xkb_nd(const Geom &g, const View<const float> &gy, const View<const float> &x, const float *k,
-                  const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws, hipStream_t s)
+                  const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws, hipStream_t s,
+                  ReduceJob *defer)
 {
     // 3D: one voxel per lane keeps the 27 gathered values per voxel and the pipeline buffers in registers
     const int vmax = knob(NDIM == 3 ? kKnobBwdkVec3d : kKnobBwdkVec2d, NDIM == 3 ? 1 : 4);
     int v = choose_vec<NDIM>(g, vmax, gy, x, gx);
     if (v == 0) v = choose_vec<NDIM>(g, 4, gy, x, gx);
     if constexpr (NDIM == 2) {
-        if (v == 4) return pick_ncb<2, 4>(g, gy, x, k, gx, pm, gk, gb, ws, s);
+        if (v == 4) return pick_ncb<2, 4>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
     }
-    if (v == 2) return pick_ncb<NDIM, 2>(g, gy, x, k, gx, pm, gk, gb, ws, s);
-    if (v == 1) return pick_ncb<NDIM, 1>(g, gy, x, k, gx, pm, gk, gb, ws, s);
+    if (v == 2) return pick_ncb<NDIM, 2>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
+    if (v == 1) return pick_ncb<NDIM, 1>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
     return hipErrorInvalidConfiguration;
 }
 

@@ -50,6 +50,7 @@ enum Knob {
     kKnobBwdxVec2d, kKnobBwdxVec3d, kKnobBwdxUnroll2d, kKnobBwdxUnroll3d, kKnobBwdxMinBlocks,
     kKnobXcdRemap, kKnobBwdkVec2d, kKnobBwdkVec3d, kKnobBwdkBlocks,
     kKnobFwdVec2d, kKnobFwdVec3d, kKnobFwdSplit, kKnobFwdRows2d, kKnobBwdkRows, kKnobBlockFuse,
+    kKnobBlockDefer,
     kKnobCount
 };
 int knob(Knob k, int dflt);
@@ -130,19 +131,33 @@ inline hipError_t fast_backward_kb(const Geom &g, bool relu, const View<const fl
                        : fast_backward_kb_2d(g, relu, out, gy, x, gk, gb, ws, s);
 }
 
+// A column reduction that has not been launched yet: `rows` partial sums per column, laid
+// out part[column][kMaxPartialRows]; columns [0, nk) accumulate into gk, the rest into gb.
+struct ReduceJob {
+    const float *part;
+    float *gk, *gb;
+    int64_t nk, ncols;
+    int rows;
+};
+constexpr int kReduceBatch = 16;
+// One launch for up to kReduceBatch pending reductions; every column is added in the same
+// order as by a launch of its own, so the sums are the same bits.
+hipError_t reduce_columns_batch(const ReduceJob *jobs, int n, hipStream_t s);
+
 // backward_x and backward_k (+ bias) of one layer in one pass (one output channel, the
 // ReLU mask already applied to gy); gk must not be null, gb may be.  Same workspace as
-// fast_backward_kb.
+// fast_backward_kb.  With `defer` the partial sums are left in the workspace and the
+// reduction that finishes gk / gb is described there instead of being launched.
 bool fast_backward_xkb_supported_2d(const Geom &g, const View<const float> &gy, const View<const float> &x,
                                     const View<float> &gx);
 bool fast_backward_xkb_supported_3d(const Geom &g, const View<const float> &gy, const View<const float> &x,
                                     const View<float> &gx);
 hipError_t fast_backward_xkb_2d(const Geom &g, const View<const float> &gy, const View<const float> &x, const float *k,
                                 const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws,
-                                hipStream_t s);
+                                hipStream_t s, ReduceJob *defer);
 hipError_t fast_backward_xkb_3d(const Geom &g, const View<const float> &gy, const View<const float> &x, const float *k,
                                 const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws,
-                                hipStream_t s);
+                                hipStream_t s, ReduceJob *defer);
 
 inline bool fast_backward_xkb_supported(const Geom &g, const View<const float> &gy, const View<const float> &x,
                                         const View<float> &gx)
@@ -151,10 +166,10 @@ inline bool fast_backward_xkb_supported(const Geom &g, const View<const float> &
 }
 inline hipError_t fast_backward_xkb(const Geom &g, const View<const float> &gy, const View<const float> &x,
                                     const float *k, const View<float> &gx, const PostMask &pm, float *gk, float *gb,
-                                    float *ws, hipStream_t s)
+                                    float *ws, hipStream_t s, ReduceJob *defer = nullptr)
 {
-    return g.ndim == 3 ? fast_backward_xkb_3d(g, gy, x, k, gx, pm, gk, gb, ws, s)
-                       : fast_backward_xkb_2d(g, gy, x, k, gx, pm, gk, gb, ws, s);
+    return g.ndim == 3 ? fast_backward_xkb_3d(g, gy, x, k, gx, pm, gk, gb, ws, s, defer)
+                       : fast_backward_xkb_2d(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
 }
 
 }  // namespace msd

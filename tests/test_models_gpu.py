@@ -99,6 +99,36 @@ def test_fused_block_backward_matches_oracle(ndim, size, c_in, depth, batch, dil
     assert max(rel_err(a, b) for a, b in zip(results[1][2], results[0][2])) <= 1e-5
 
 
+@pytest.mark.parametrize("ndim,size,depth", [(2, (24, 128), 37), (3, (5, 6, 64), 19)])
+def test_block_backward_deferred_reductions_give_the_same_bits(ndim, size, depth):
+    # the reverse loop reduces the partial weight-gradient sums of up to 16 layers in one
+    # launch; every column is added in the order a launch of its own uses
+    from msd_pytorch_amd import _native
+    from msd_pytorch_amd import msd_custom_convolutions as cc
+    x, dil, bias, ws, g = make_block_problem(ndim, size, 2, 1, depth, torch.float32, batch=2)
+    lib = _native.load()
+    stack = torch.empty(2, 2 + depth, *size, device="cuda")
+    stack[:, :2] = x.cuda()
+    wd = [w.cuda() for w in ws]
+    cc.block_forward(stack, 2, dil, bias.cuda(), wd)
+    results = []
+    for defer in (1, 0):
+        assert lib.msd_set_tuning(b"block.defer", defer) == 0
+        try:
+            grads = g.cuda().clone()
+            gw = [torch.zeros_like(w) for w in wd]
+            gb = torch.zeros(depth, device="cuda")
+            cc.block_backward(stack, grads, 2, dil, wd, gw, gb, True)
+            torch.cuda.synchronize()
+        finally:
+            lib.msd_set_tuning(b"block.defer", -1)
+        results.append((grads[:, :2].clone(), gb, gw))
+    assert torch.equal(results[0][0], results[1][0])
+    assert torch.equal(results[0][1], results[1][1])
+    assert all(torch.equal(a, b) for a, b in zip(results[0][2], results[1][2]))
+    assert all(float(w.abs().max()) > 0 for w in results[0][2])
+
+
 def test_depth_100_stack_stays_within_tolerance():
     # errors compound through the layers: the full depth of the headline network on a small image
     from msd_pytorch_amd.msd_block import msd_block
