@@ -205,12 +205,11 @@ def main():
     model.set_input(x)          # inputs resident in HBM before the timed region
     model.set_target(target)
 
+    # one batch of MSDModel.train: forward, zero_grad, backward and, where the workload has
+    # it, the Adam update, on the batch resident in HBM; like train, the loop does not read
+    # the loss back between steps
     def step():
-        model.forward()
-        model.optimizer.zero_grad()
-        model.loss.backward()
-        if adam:
-            model.optimizer.step()
+        model.step_async(update=adam)
 
     for _ in range(args.warmup):
         step()

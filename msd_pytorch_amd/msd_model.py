@@ -6,13 +6,36 @@ import torch
 import torch.nn as nn
 import torch.optim as optim
 
-from .msd_module import MSDModule
+from . import msd_custom_convolutions as cc
+from .msd_module import MSDFinalFunction, MSDModule
+
+
+class _NativePointwise:
+    """forward of a 1x1 convolution as one native pass over the voxels (the kernel of the
+    network's final layer) for GPU tensors with contiguous channel planes; torch's
+    convolution otherwise.  Parameters, state-dict keys and initialisation are those of
+    the torch class it is mixed into."""
+
+    def forward(self, input):
+        w = self.weight
+        if self.bias is not None and input.dim() == w.dim() and input.dtype == w.dtype \
+                and w.is_cuda and cc.final_layer_supported(input):
+            return MSDFinalFunction.apply(input, w.view(w.shape[0], w.shape[1]), self.bias)
+        return super().forward(input)
+
+
+class ScalingConv2d(_NativePointwise, nn.Conv2d):
+    pass
+
+
+class ScalingConv3d(_NativePointwise, nn.Conv3d):
+    pass
 
 
 def scaling_module(num_channels, *, conv3d=False):
     """A frozen 1x1 convolution initialised to the identity.  It is saved with
     the network and never touched by the optimiser."""
-    conv = nn.Conv3d if conv3d else nn.Conv2d
+    conv = ScalingConv3d if conv3d else ScalingConv2d
     c = conv(num_channels, num_channels, 1)
     c.bias.requires_grad = False
     c.weight.requires_grad = False
@@ -112,8 +135,8 @@ class MSDModel:
         assert self.c_out == data.shape[1], "Wrong number of output channels"
         self.target = data.cuda()
 
-    def forward(self, input=None, target=None):
-        """Loss of one (input, target) pair; arguments left out keep their last value."""
+    def _launch_forward(self, input=None, target=None):
+        """Network and criterion on one (input, target) pair, without waiting for the GPU."""
         if input is not None:
             self.set_input(input)
         if target is not None:
@@ -122,20 +145,40 @@ class MSDModel:
         self.loss = None
         self.output = self.net(self.input)
         self.loss = self.criterion(self.output, self.target)
+
+    def forward(self, input=None, target=None):
+        """Loss of one (input, target) pair; arguments left out keep their last value."""
+        self._launch_forward(input, target)
+        return self.loss.item()
+
+    def step_async(self, input=None, target=None, update=True):
+        """Launch forward, zero_grad, backward and (``update``) the optimiser step of
+        msd_model.py:225-244 without waiting for the GPU.  Nothing is returned: ``get_loss()``
+        reads the loss when it is wanted, and waits then."""
+        self._launch_forward(input, target)
+        self.optimizer.zero_grad()
+        self.loss.backward()
+        if update:
+            self.optimizer.step()
+
+    def gradients(self, input=None, target=None):
+        """forward + zero_grad + backward: what ``learn`` does short of the optimiser step.
+        Returns the loss."""
+        self.step_async(input, target, update=False)
         return self.loss.item()
 
     def learn(self, input=None, target=None):
-        """One optimisation step on one (input, target) pair; returns the loss."""
-        loss = self.forward(input, target)
-        self.optimizer.zero_grad()
-        self.loss.backward()
-        self.optimizer.step()
-        return loss
+        """One optimisation step on one (input, target) pair; returns the loss (read back
+        after the whole step has been launched)."""
+        self.step_async(input, target)
+        return self.loss.item()
 
     def train(self, dataloader, num_epochs):
+        # the loss of each batch is not looked at here (msd_model.py:246-261 drops it too):
+        # the host keeps launching ahead of the GPU
         for _ in range(num_epochs):
             for input, target in dataloader:
-                self.learn(input, target)
+                self.step_async(input, target)
 
     def validate(self, dataloader):
         """Mean loss per (input, target) pair of the loader."""

@@ -330,6 +330,50 @@ def test_getting_started_example(task, tmp_path):
         assert float(outputs[0].max()) <= 2
 
 
+@pytest.mark.parametrize("ndim,channels", [(2, 1), (2, 3), (3, 2)])
+def test_scaling_modules_run_natively_and_match_conv(ndim, channels):
+    # scale_in / scale_out (msd_model.py:8-45) are nn.Conv2d/3d subclasses whose forward is one
+    # native pass on the GPU; values and input gradient are those of the torch convolution
+    from msd_pytorch_amd.msd_model import scaling_module, scaling_module_set_bias, scaling_module_set_scale
+    torch.manual_seed(5)
+    sm = scaling_module(channels, conv3d=ndim == 3).cuda()
+    assert isinstance(sm, torch.nn.Conv3d if ndim == 3 else torch.nn.Conv2d)
+    assert sorted(sm.state_dict()) == ["bias", "weight"]
+    scaling_module_set_scale(sm, 0.37)
+    scaling_module_set_bias(sm, -1.25)
+    sm.weight.data += 0.01 * torch.randn_like(sm.weight)      # off-diagonal terms too
+    size = (19, 70) if ndim == 2 else (5, 9, 34)
+    x = torch.randn(2, channels, *size, device="cuda", requires_grad=True)
+    g = torch.randn(2, channels, *size, device="cuda")
+    y = sm(x)
+    y.backward(g)
+    conv = torch.nn.functional.conv3d if ndim == 3 else torch.nn.functional.conv2d
+    x2 = x.detach().clone().requires_grad_(True)
+    y2 = conv(x2, sm.weight, sm.bias)
+    y2.backward(g)
+    assert rel_err(y, y2) <= 1e-6 and rel_err(x.grad, x2.grad) <= 1e-6
+    assert sm.weight.grad is None and sm.bias.grad is None
+    # a view with strided planes falls back to torch
+    xs = torch.randn(2, channels, *size[:-1], 2 * size[-1], device="cuda")[..., ::2]
+    assert rel_err(sm(xs), conv(xs, sm.weight, sm.bias)) <= 1e-6
+
+
+def test_gradients_and_learn_report_the_forward_loss():
+    from msd_pytorch_amd import MSDRegressionModel
+    torch.manual_seed(2)
+    model = MSDRegressionModel(1, 1, depth=4, width=1, dilations=[1, 2])
+    model.msd.final_layer.linear.weight.data.normal_(0, 0.1)
+    x = torch.randn(1, 1, 24, 40)
+    y = 0.5 * x
+    loss = model.forward(x, y)
+    assert model.gradients(x, y) == loss
+    grads = [p.grad.clone() for p in model.msd.parameters()]
+    assert all(g is not None and bool(torch.isfinite(g).all()) for g in grads)
+    assert any(float(g.abs().max()) > 0 for g in grads)
+    assert model.learn(x, y) == loss                           # the loss before the update
+    assert model.forward(x, y) != loss                         # the update moved the parameters
+
+
 def test_regression_state_dict_keys():
     # key layout of the reference's checkpoints (msd_regression_model.py:76, msd_block.py:170-179)
     from msd_pytorch_amd import MSDRegressionModel
