@@ -58,6 +58,7 @@ struct Args {
     Geom g;
     RowTeams rt;
     int remap, tiles_per_wg, ngroups, total_groups;
+    int group_step;      // 1: a workgroup walks consecutive row groups; > 1: every group_step-th one
     Plane gy;            // masked output gradient, one channel (sc unused)
     Plane x;             // input channels
     Plane gx;            // grad_input channels (written through a cast)
@@ -113,7 +114,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_rows_fused(const Args a, cons
 
     // Position of the lane's row, advanced from tile to tile without divisions: the row groups
     // of a workgroup are consecutive.
-    int grp = lb * a.tiles_per_wg;
+    int grp = a.group_step == 1 ? lb * a.tiles_per_wg : lb;
     int gi = grp % a.ngroups, b = grp / a.ngroups;            // uniform: group within the image, batch index
     int row = gi * rt.rpw + team;
     int y = row % g.H, z = row / g.H;
@@ -311,6 +312,15 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_rows_fused(const Args a, cons
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         // next row group
+        if (a.group_step != 1) {                  // uniform
+            grp += a.group_step;
+            gi = grp % a.ngroups;
+            b = grp / a.ngroups;
+            row = gi * rt.rpw + team;
+            y = row % g.H;
+            z = row / g.H;
+            continue;
+        }
         grp++;
         if (++gi == a.ngroups) {                  // uniform: first group of the next batch item
             gi = 0;
@@ -417,6 +427,13 @@ hipError_t launch(const Geom &g, const View<const float> &gy, const View<const f
     const int64_t wgs = (total + a.tiles_per_wg - 1) / a.tiles_per_wg;
     const int rows = a.remap ? xcd_grid((int)wgs) : (int)wgs;   // padding workgroups write zero rows
     if (rows > kMaxPartialRows || total > INT32_MAX) return hipErrorInvalidConfiguration;
+    a.group_step = 1;
+    if (knob(kKnobBwdkInterleave, 1) && total + rows < INT32_MAX) {
+        // the workgroups sweep the image together: at any time they work on one window of
+        // consecutive rows, every workgroup on every rows-th group
+        a.group_step = rows;
+        a.tiles_per_wg = (int)((total + rows - 1) / rows);
+    }
     a.total_groups = (int)total;
     a.gy = Plane{(int)gy.sb, (int)gy.sc, (int)gy.sz, (int)gy.sy};
     a.x = Plane{(int)x.sb, (int)x.sc, (int)x.sz, (int)x.sy};

@@ -66,6 +66,8 @@ def test_block_matches_oracle(ndim, size, c_in, width, depth, dtype):
     (3, (9, 11, 128), 1, 18, 1, None),     # one voxel per lane, 2 rows per workgroup
     (3, (6, 7, 68), 2, 6, 2, None),        # 68 of 128 lanes per row busy
     (3, (12, 5, 64), 1, 3, 1, [5, 1, 4]),  # dilation == smallest extent
+    (2, (700, 260), 1, 3, 2, None),        # more row groups than workgroups: several tiles each
+    (3, (33, 31, 68), 2, 3, 2, None),      # the same in 3D, last groups ragged
 ])
 def test_fused_block_backward_matches_oracle(ndim, size, c_in, depth, batch, dilations):
     from msd_pytorch_amd import _native
