@@ -297,7 +297,18 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_rows_fused(const Args a, cons
             for (int tg = 0; tg < TG; tg++) acc[tg][0] = acc[tg][1] = mfma4{0.f, 0.f, 0.f, 0.f};
             stage_k(cb, h, ka);
             stage_x(cb, h, ga);
-            if (st + 2 < nst) load_stage((st + 2) / H, (st + 2) % H, ka, ga);
+            // 2D: no test around these loads.  Loads and stores retire through one in-order
+            // counter and the compiler derives each wait from what may be pending on any path,
+            // so a load that may be skipped turns the wait in front of the next matrix
+            // instructions into one for these loads themselves.  The last iteration loads its
+            // own first stage again instead (cache hits, never used).  Measured: 2 % faster in
+            // 2D, 2 % slower in 3D (fewer, longer iterations per tile), which keeps the test.
+            if constexpr (NDIM == 2) {
+                const int sn = min(st + 2, nst - 2);
+                load_stage(sn / H, sn % H, ka, ga);
+            } else {
+                if (st + 2 < nst) load_stage((st + 2) / H, (st + 2) % H, ka, ga);
+            }
             stage_k(cb, h + 1, kb);
             stage_x(cb, h + 1, gb);
             // D is indexed statically: pick the block with a chain of uniform branches
