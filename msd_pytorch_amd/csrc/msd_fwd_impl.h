@@ -293,7 +293,11 @@ hipError_t pick(const Geom &g, const View<const float> &x, const float *k, const
             if (best == 5) return launch<2, RELU, 1, 4, 1, 5>(g, x, k, bias, out, s);
             if (best == 6) return launch<2, RELU, 1, 4, 1, 6>(g, x, k, bias, out, s);
         }
-        if (v == 4) return launch<2, RELU, WOUT, 4, 1, 4>(g, x, k, bias, out, s);
+        // two output channels double the accumulators: three rows per tile keep them in registers
+        if (v == 4 && WOUT == 2) return launch<2, RELU, 2, 4, 1, 3>(g, x, k, bias, out, s);
+        if constexpr (WOUT == 1) {
+            if (v == 4) return launch<2, RELU, 1, 4, 1, 4>(g, x, k, bias, out, s);
+        }
         if (v == 2) return launch<2, RELU, WOUT, 2, 1, 4>(g, x, k, bias, out, s);
         if (v == 1) return launch<2, RELU, WOUT, 1, 1, 4>(g, x, k, bias, out, s);
     }
