@@ -174,6 +174,8 @@ def main():
     ap.add_argument("--no-kernel-timing", action="store_true")
     ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
                     help="launch-shape knob passed to msd_set_tuning (repeatable)")
+    ap.add_argument("--graph", action="store_true",
+                    help="replay the step from a HIP graph (GraphedStep): for workloads bound by launch overhead")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run one 1 GiB device copy first (reference dispatch for scaling rocprof byte counters)")
     args = ap.parse_args()
@@ -211,6 +213,13 @@ def main():
     def step():
         model.step_async(update=adam)
 
+    eager_step = step
+    if args.graph:
+        from msd_pytorch_amd import GraphedStep
+        if adam:
+            model.optimizer = torch.optim.Adam(model.msd.parameters(), capturable=True)
+        step = GraphedStep(model, update=adam)    # the per-kernel timing below runs the eager step
+
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -231,11 +240,11 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"{name}: {DESCRIPTION[name]}", "depth": depth, "width": width,
-                   "batch": batch, "spatial": list(spatial)},
+                   "batch": batch, "spatial": list(spatial), "hip_graph": bool(args.graph)},
     }
 
     if not args.no_kernel_timing:
-        totals = kernel_times(lib, torch, lambda: [step() for _ in range(args.steps)])
+        totals = kernel_times(lib, torch, lambda: [eager_step() for _ in range(args.steps)])
         bytes_per_step, _ = algorithmic_bytes(name, totals["backward_xkb"][1] > 0)
         kernels = {}
         for cls, (ms, launches) in totals.items():

@@ -10,6 +10,7 @@ from .msd_block import MSDBlock, MSDBlock2d, MSDBlock3d, MSDBlockFunction, msd_b
 from .msd_module import MSDFinalLayer, MSDModule  # noqa: E402,F401
 from .errors import Error, InputError  # noqa: E402,F401
 from .image_dataset import ImageDataset, ImageStack  # noqa: E402,F401
+from .msd_model import GraphedStep  # noqa: E402,F401
 from .msd_regression_model import MSDRegressionModel  # noqa: E402,F401
 from .msd_segmentation_model import MSDSegmentationModel  # noqa: E402,F401
 

@@ -93,6 +93,64 @@ def match_module_prefix(state_dict, wanted_keys):
     return type(state_dict)(("module." + k, v) for k, v in state_dict.items())
 
 
+class GraphedStep:
+    """One train step of an MSDModel recorded as a HIP graph and replayed.
+
+    ``GraphedStep(model)`` runs ``model.step_async(update=update)`` a few times on the
+    model's current input and target (set them first with ``set_input`` / ``set_target``),
+    then captures one more run.  Calling the object copies a new input and target (when
+    given; same shapes) into the captured buffers and replays the whole step, scaling
+    layers, loss and backward pass included, as a single launch: what a network this small
+    needs, since its step is otherwise bound by launch overhead, not by the kernels.
+    ``loss()`` reads the loss of the last replay; the parameters' ``.grad`` hold its
+    gradients.  With ``update=True`` the optimiser step is part of the graph, which torch
+    only allows for an optimiser built with ``capturable=True``
+    (``model.optimizer = torch.optim.Adam(params, capturable=True)``); the ``warmup`` runs
+    (at least one) are then real optimisation steps on the current batch, and they are what
+    creates the optimiser's state outside the graph.
+
+    The captured work is the eager work, launch for launch, so replays give the same bits."""
+
+    def __init__(self, model, update=False, warmup=3):
+        if update and not model.optimizer.defaults.get("capturable", False):
+            raise ValueError("GraphedStep(update=True) needs an optimiser built with capturable=True")
+        if update and warmup < 1:
+            raise ValueError("GraphedStep(update=True) needs warmup >= 1: the optimiser creates its state in its "
+                             "first step, which must not be part of the graph")
+        if getattr(model, "input", None) is None or getattr(model, "target", None) is None:
+            raise ValueError("GraphedStep: call set_input and set_target first")
+        self.model = model
+        model.loss = model.output = None          # no autograd graph of an earlier step kept alive
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(warmup):
+                model.step_async(update=update)
+        torch.cuda.current_stream().wait_stream(side)
+        model.optimizer.zero_grad(set_to_none=True)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            model.step_async(update=update)
+        self._input, self._target = model.input, model.target
+        self._loss, self._output = model.loss, model.output
+        # the gradient tensors the graph writes (an eager step in between replaces .grad)
+        self._grads = [(p, p.grad) for group in model.optimizer.param_groups for p in group["params"]
+                       if p.grad is not None]
+
+    def __call__(self, input=None, target=None):
+        if input is not None:
+            self._input.copy_(input, non_blocking=True)
+        if target is not None:
+            self._target.copy_(target.reshape(self._target.shape), non_blocking=True)
+        self.graph.replay()
+        self.model.loss, self.model.output = self._loss, self._output
+        for p, g in self._grads:
+            p.grad = g
+
+    def loss(self):
+        return self._loss.item()
+
+
 class MSDModel:
     """Base class; use MSDRegressionModel or MSDSegmentationModel.
 

@@ -376,6 +376,69 @@ def test_gradients_and_learn_report_the_forward_loss():
     assert model.forward(x, y) != loss                         # the update moved the parameters
 
 
+@pytest.mark.parametrize("kind,ndim", [("regression", 2), ("segmentation", 2), ("regression", 3)])
+def test_step_replayed_from_a_hip_graph_equals_the_eager_step(kind, ndim):
+    # every replay is checked against the eager step on the same data, with eager work and
+    # synchronisations between the replays
+    from msd_pytorch_amd import GraphedStep, MSDRegressionModel, MSDSegmentationModel
+    torch.manual_seed(11)
+    size = (48, 96) if ndim == 2 else (6, 10, 64)
+    dil = [1, 2, 3, 4, 5]
+    if kind == "regression":
+        model = MSDRegressionModel(2, 1, depth=9, width=1, dilations=dil, ndim=ndim)
+        new_target = lambda: torch.randn(2, 1, *size)
+    else:
+        model = MSDSegmentationModel(2, 3, depth=9, width=1, dilations=dil, ndim=ndim)
+        new_target = lambda: torch.randint(0, 3, (2, 1, *size))
+    model.msd.final_layer.linear.weight.data.normal_(0, 0.2)
+    model.set_input(torch.randn(2, 2, *size))
+    model.set_target(new_target())
+    params = list(model.msd.parameters())
+    graphed = GraphedStep(model)
+    for _ in range(3):
+        x, t = torch.randn(2, 2, *size), new_target()
+        graphed(x, t)
+        got = [torch.tensor(graphed.loss())] + [p.grad.detach().clone().cpu() for p in params]
+        assert model.get_loss() == graphed.loss() and model.get_output().shape[0] == 2
+        eager_loss = model.gradients(x, t)
+        want = [torch.tensor(eager_loss)] + [p.grad.detach().clone().cpu() for p in params]
+        assert all(torch.equal(a, b) for a, b in zip(got, want))
+        assert all(float(g.abs().max()) > 0 for g in got[1:])
+    with pytest.raises(ValueError, match="capturable"):
+        GraphedStep(model, update=True)
+
+
+def test_graphed_step_with_capturable_adam_follows_the_eager_optimiser():
+    from msd_pytorch_amd import GraphedStep, MSDRegressionModel
+    size = (32, 64)
+    models = []
+    for _ in range(2):
+        torch.manual_seed(12)
+        m = MSDRegressionModel(1, 1, depth=6, width=1, dilations=[1, 2, 3])
+        m.msd.final_layer.linear.weight.data.normal_(0, 0.2)
+        m.optimizer = torch.optim.Adam(m.msd.parameters(), capturable=True)
+        models.append(m)
+    eager, captured = models
+    torch.manual_seed(13)
+    batches = [(torch.randn(1, 1, *size), torch.randn(1, 1, *size)) for _ in range(4)]
+    captured.set_input(batches[0][0])
+    captured.set_target(batches[0][1])
+    with pytest.raises(ValueError, match="warmup"):
+        GraphedStep(captured, update=True, warmup=0)
+    graphed = GraphedStep(captured, update=True, warmup=1)     # one real step on the first batch
+    eager.learn(*batches[0])
+    before = [p.detach().clone() for p in captured.msd.parameters()]
+    for p, q in zip(captured.msd.parameters(), eager.msd.parameters()):
+        assert rel_err(p.detach(), q.detach()) <= 1e-6         # the capture itself records, it does not run
+    for x, t in batches[1:]:
+        graphed(x, t)
+        eager.learn(x, t)
+        assert abs(graphed.loss() - eager.get_loss()) <= 1e-6 * max(1.0, abs(eager.get_loss()))
+    for a, b in zip(captured.msd.parameters(), eager.msd.parameters()):
+        assert rel_err(a.detach(), b.detach()) <= 1e-5
+    assert any(not torch.equal(p.detach(), b) for p, b in zip(captured.msd.parameters(), before))
+
+
 def test_regression_state_dict_keys():
     # key layout of the reference's checkpoints (msd_regression_model.py:76, msd_block.py:170-179)
     from msd_pytorch_amd import MSDRegressionModel
