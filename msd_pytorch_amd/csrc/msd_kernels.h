@@ -50,10 +50,13 @@ enum Knob {
     kKnobBwdxVec2d, kKnobBwdxVec3d, kKnobBwdxUnroll2d, kKnobBwdxUnroll3d, kKnobBwdxMinBlocks,
     kKnobXcdRemap, kKnobBwdkVec2d, kKnobBwdkVec3d, kKnobBwdkBlocks,
     kKnobFwdVec2d, kKnobFwdVec3d, kKnobFwdSplit, kKnobFwdRows2d, kKnobBwdkRows, kKnobBlockFuse,
-    kKnobBlockDefer, kKnobBwdkInterleave,
+    kKnobBlockDefer, kKnobBwdkInterleave, kKnobBlockSnake,
     kKnobCount
 };
 int knob(Knob k, int dflt);
+// Set by the dense block's layer loops: walk the input channels from the last to the first
+// in the next launches (see msd_block_forward).
+bool reverse_channels();
 extern const char *const kKnobNames[kKnobCount];
 extern int g_knobs[kKnobCount];
 
