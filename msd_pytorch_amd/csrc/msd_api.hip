@@ -617,8 +617,11 @@ int block_layer_fused(const char *fn, const BlockArgs &a, int i, int64_t first, 
     msd::ReduceJob *job = nullptr;
     MSD_TRY(pending->next(fn, region, &job));
     ProfileScope scope(3, s);
+    // as in the forward loop: alternate layers walk the channels in opposite directions
+    msd::g_reverse_channels = msd::knob(msd::kKnobBlockSnake, 1) && (i & 1);
     const hipError_t e = msd::fast_backward_xkb(g, gy, x, (const float *)weights_i, gx, pm, (float *)gk, (float *)gb,
                                                 (float *)ws, s, job);
+    msd::g_reverse_channels = false;
     if (e != hipSuccess) return hip_fail(fn, e);
     if (job) pending->taken(region);
     *done = true;

@@ -59,6 +59,7 @@ struct Args {
     RowTeams rt;
     int remap, tiles_per_wg, ngroups, total_groups;
     int group_step;      // 1: a workgroup walks consecutive row groups; > 1: every group_step-th one
+    int reverse;         // walk the blocks of 16 channels from the last to the first
     Plane gy;            // masked output gradient, one channel (sc unused)
     Plane x;             // input channels
     Plane gx;            // grad_input channels (written through a cast)
@@ -160,7 +161,9 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_rows_fused(const Args a, cons
                 load_global_vec<V>(channel_base(gbase, ci), goff, gg[j]);
             }
         };
-        load_stage(0, 0, ka, ga);   // issued ahead of the gather so the two latencies overlap
+        // block of 16 channels that stage `s` of the walk belongs to
+        auto block_of = [&](int s) { return a.reverse ? ncb - 1 - s / H : s / H; };
+        load_stage(block_of(0), 0, ka, ga);   // issued ahead of the gather so the two latencies overlap
 
         // ---- A operands, voxel layout: tv[t][i] = A[t](voxel x0 + i of the team's row)
         float tv[K][V];
@@ -291,7 +294,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_rows_fused(const Args a, cons
         const int nst = ncb * H;                  // even
 #pragma unroll 1
         for (int st = 0; st < nst; st += 2) {
-            const int cb = st / H, h = st % H;
+            const int cb = block_of(st), h = st % H;
             load_stage(cb, h + 1, kb, gb);
 #pragma unroll
             for (int tg = 0; tg < TG; tg++) acc[tg][0] = acc[tg][1] = mfma4{0.f, 0.f, 0.f, 0.f};
@@ -305,9 +308,9 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_rows_fused(const Args a, cons
             // 2D, 2 % slower in 3D (fewer, longer iterations per tile), which keeps the test.
             if constexpr (NDIM == 2) {
                 const int sn = min(st + 2, nst - 2);
-                load_stage(sn / H, sn % H, ka, ga);
+                load_stage(block_of(sn), sn % H, ka, ga);
             } else {
-                if (st + 2 < nst) load_stage((st + 2) / H, (st + 2) % H, ka, ga);
+                if (st + 2 < nst) load_stage(block_of(st + 2), (st + 2) % H, ka, ga);
             }
             stage_k(cb, h + 1, kb);
             stage_x(cb, h + 1, gb);
@@ -438,6 +441,7 @@ hipError_t launch(const Geom &g, const View<const float> &gy, const View<const f
     const int64_t wgs = (total + a.tiles_per_wg - 1) / a.tiles_per_wg;
     const int rows = a.remap ? xcd_grid((int)wgs) : (int)wgs;   // padding workgroups write zero rows
     if (rows > kMaxPartialRows || total > INT32_MAX) return hipErrorInvalidConfiguration;
+    a.reverse = reverse_channels();
     a.group_step = 1;
     if (knob(kKnobBwdkInterleave, 1) && total + rows < INT32_MAX) {
         // the workgroups sweep the image together: at any time they work on one window of
