@@ -68,6 +68,14 @@ int msd_set_kernel_path(int path);
  * per lane) or "bwdx.unroll3d" (channels in flight).  value < 0 restores the
  * library default; values a kernel was not built for fall back to the default.
  * Results do not depend on these settings beyond floating-point summation order.
+ * Keys: "bwdx.vec2d", "bwdx.vec3d", "bwdk.vec2d", "bwdk.vec3d", "fwd.vec2d", "fwd.vec3d"
+ * (voxels per lane), "bwdx.unroll2d", "bwdx.unroll3d" (channels in flight),
+ * "bwdx.min_blocks", "bwdk.blocks" (workgroups per launch), "fwd.split" (channel groups
+ * per workgroup), "fwd.rows2d" (rows per forward tile), "xcd_remap" (0/1: workgroup order
+ * by XCD), "bwdk.rows" (0/1: row-team weight-gradient kernel), "bwdk.interleave" (0/1:
+ * workgroups take every n-th row group), "block.fuse" (0/1: fused backward in the block),
+ * "block.defer" (0/1: one reduction launch for many layers), "block.snake" (0/1: alternate
+ * layers walk the channels in opposite directions).  Unknown keys return MSD_ERR_INVALID.
  */
 int msd_set_tuning(const char *key, int value);
 

@@ -17,7 +17,13 @@ const char *const kKnobNames[kKnobCount] = {
     "fwd.vec2d", "fwd.vec3d", "fwd.split", "fwd.rows2d", "bwdk.rows", "block.fuse",
     "block.defer", "bwdk.interleave", "block.snake",
 };
-int g_knobs[kKnobCount] = {-1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1};
+static_assert(kKnobBlockSnake + 1 == kKnobCount, "one name per knob, in the order of the enum");
+int g_knobs[kKnobCount];
+// every knob starts at "library default"
+const bool g_knobs_ready = [] {
+    for (int i = 0; i < kKnobCount; i++) g_knobs[i] = -1;
+    return true;
+}();
 int knob(Knob k, int dflt) { return g_knobs[k] < 0 ? dflt : g_knobs[k]; }
 // per thread: callers on different threads (one per device under DataParallel) do not meet
 thread_local bool g_reverse_channels = false;

@@ -94,5 +94,13 @@ def test_tuning_hook_rejects_unknown_key():
     lib = _native.load()
     assert lib.msd_set_tuning(b"no.such.knob", 1) == _native.MSD_ERR_INVALID
     assert lib.msd_set_tuning(b"xcd_remap", -1) == _native.MSD_OK
+    # every key the header documents is known to the library
+    import re
+    header = open(os.path.join(ROOT, "include", "msd_hip.h")).read()
+    doc = header[header.index("Keys:"):header.index("Unknown keys")]
+    keys = re.findall(r'"([a-z0-9_.]+)"', doc)
+    assert len(keys) == len(set(keys)) >= 18
+    for key in keys:
+        assert lib.msd_set_tuning(key.encode(), -1) == _native.MSD_OK, key
     assert lib.msd_set_kernel_path(2) == _native.MSD_ERR_INVALID
     assert lib.msd_set_kernel_path(0) == _native.MSD_OK
