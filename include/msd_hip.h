@@ -75,7 +75,8 @@ int msd_set_kernel_path(int path);
  * by XCD), "bwdk.rows" (0/1: row-team weight-gradient kernel), "bwdk.interleave" (0/1:
  * workgroups take every n-th row group), "block.fuse" (0/1: fused backward in the block),
  * "block.defer" (0/1: one reduction launch for many layers), "block.snake" (0/1: alternate
- * layers walk the channels in opposite directions).  Unknown keys return MSD_ERR_INVALID.
+ * layers walk the channels in opposite directions), "fwd.class3d" (0/1: 3D forward tiles
+ * numbered by residue class).  Unknown keys return MSD_ERR_INVALID.
  */
 int msd_set_tuning(const char *key, int value);
 

@@ -39,6 +39,7 @@ struct Lattice {
     int tiles_z;    // dil * segs_z (1 in 2D)
     int ntiles;
     int reverse;    // walk the input channels from the last to the first
+    int by_class;   // 3D: tiles numbered residue class by residue class (2: a class row by row, no blocks)
 };
 
 template <int NDIM, bool RELU, int WOUT, int V, int RZ, int RY>
@@ -59,7 +60,28 @@ __global__ __launch_bounds__(1024) void fwd_lattice(Geom g, Lattice lt, int rema
     // lattices share a third of their input rows, and only tiles that start together walk the
     // channels in step and find each other's rows in the L2.
     int ty, tz;
-    if (NDIM == 3) {
+    if (NDIM == 3 && lt.by_class == 2) {
+        // small classes (large dilations): all lattices of a class are resident together
+        // anyway, so they are simply numbered row by row, with no padding of the grid
+        const int per_class = lt.segs_y * lt.segs_z;
+        const int cls = tile / per_class, rem = tile % per_class;
+        ty = (cls % g.dil) * lt.segs_y + rem % lt.segs_y;
+        tz = (cls / g.dil) * lt.segs_z + rem / lt.segs_y;
+    } else if (NDIM == 3 && lt.by_class) {
+        // An input row feeds only output rows of its own residue class (y mod dil, z mod dil):
+        // the lattices of one class share all their input, those of different classes nothing.
+        // So the classes are numbered one after the other, and inside a class the lattices in
+        // blocks of kOrder x kOrder neighbours: what runs together, on one XCD, reads the same
+        // rows, and the L2 serves the re-reads.
+        const int bys = (lt.segs_y + kOrder - 1) / kOrder, bzs = (lt.segs_z + kOrder - 1) / kOrder;
+        const int per_class = bys * bzs * kOrder * kOrder;
+        const int cls = tile / per_class, rem = tile % per_class;
+        const int blk = rem / (kOrder * kOrder), within = rem % (kOrder * kOrder);
+        const int sy = (blk % bys) * kOrder + within % kOrder, sz = (blk / bys) * kOrder + within / kOrder;
+        if (sy >= lt.segs_y || sz >= lt.segs_z) return;     // padding of the block grid (whole workgroup)
+        ty = (cls % g.dil) * lt.segs_y + sy;
+        tz = (cls / g.dil) * lt.segs_z + sz;
+    } else if (NDIM == 3) {
         const int blk = tile / (kOrder * kOrder), within = tile % (kOrder * kOrder);
         const int nby = (lt.tiles_y + kOrder - 1) / kOrder;
         ty = (blk % nby) * kOrder + within % kOrder;
@@ -222,8 +244,17 @@ inline bool make_lattice(const Geom &g, int V, int rz, int ry, int ks_wanted, La
     if (g.ndim == 3) {
         lt->segs_z = ((g.D + g.dil - 1) / g.dil + rz - 1) / rz;
         lt->tiles_z = g.dil * lt->segs_z;
-        lt->ntiles = ((lt->tiles_y + kOrder - 1) / kOrder) * ((lt->tiles_z + kOrder - 1) / kOrder) * kOrder * kOrder;
+        lt->by_class = knob(kKnobFwdClass3d, 1);
+        if (lt->by_class && lt->segs_y * lt->segs_z <= 128) lt->by_class = 2;
+        if (lt->by_class == 2)
+            lt->ntiles = g.dil * g.dil * lt->segs_y * lt->segs_z;
+        else if (lt->by_class)
+            lt->ntiles = g.dil * g.dil * ((lt->segs_y + kOrder - 1) / kOrder) * ((lt->segs_z + kOrder - 1) / kOrder) *
+                         kOrder * kOrder;
+        else
+            lt->ntiles = ((lt->tiles_y + kOrder - 1) / kOrder) * ((lt->tiles_z + kOrder - 1) / kOrder) * kOrder * kOrder;
     } else {
+        lt->by_class = 0;
         lt->segs_z = 1;
         lt->tiles_z = 1;
         lt->ntiles = lt->tiles_y;
