@@ -101,22 +101,24 @@ __global__ __launch_bounds__(1024) void fwd_lattice(Geom g, Lattice lt, int rema
     const bool act = lane * V < g.W;
     const int b = blockIdx.y;
 
-    // Offsets of the input lattice rows (fold, then clamp rows that only feed output rows
-    // outside the image).  A load address is a wave-uniform base (batch, channel, z level:
-    // scalar registers and scalar arithmetic) plus a 32-bit byte offset per lane (y row and
-    // x position, computed once), so the channel loop spends no vector instructions on it.
+    // valid output rows of this lattice (the rest lie past the image edge)
+    const int nyv = min(RY, (g.H - y0 + g.dil - 1) / g.dil);
+    const int nzv = NDIM == 3 ? min(RZ, (g.D - z0 + g.dil - 1) / g.dil) : 1;
+
+    // Offsets of the input lattice rows (folded at the image edges).  Lattice levels past
+    // nyv + 1 (nzv + 1) feed only output rows outside the image: they repeat the last level
+    // that is needed, so that their loads hit the cache instead of fetching rows nobody uses.
+    // A load address is a wave-uniform base (batch, channel, z level: scalar registers and
+    // scalar arithmetic) plus a 32-bit byte offset per lane (y row and x position, computed
+    // once), so the channel loop spends no vector instructions on it.
     int64_t offz[LZ];
     uint32_t offyx[LY];
 #pragma unroll
     for (int m = 0; m < LZ; m++)
-        offz[m] = NDIM == 3 ? (int64_t)min(reflect_idx(min(z0 + (m - 1) * g.dil, 2 * g.D - 1), g.D), g.D - 1) * x.sz * 4 : 0;
+        offz[m] = NDIM == 3 ? (int64_t)min(reflect_idx(min(z0 + (min(m, nzv + 1) - 1) * g.dil, 2 * g.D - 1), g.D), g.D - 1) * x.sz * 4 : 0;
 #pragma unroll
     for (int m = 0; m < LY; m++)
-        offyx[m] = 4u * (uint32_t)(min(reflect_idx(min(y0 + (m - 1) * g.dil, 2 * g.H - 1), g.H), g.H - 1) * (int)x.sy + x0);
-
-    // valid output rows of this lattice (the rest lie past the image edge)
-    const int nyv = min(RY, (g.H - y0 + g.dil - 1) / g.dil);
-    const int nzv = NDIM == 3 ? min(RZ, (g.D - z0 + g.dil - 1) / g.dil) : 1;
+        offyx[m] = 4u * (uint32_t)(min(reflect_idx(min(y0 + (min(m, nyv + 1) - 1) * g.dil, 2 * g.H - 1), g.H), g.H - 1) * (int)x.sy + x0);
 
     float acc[WOUT][RZ][RY][3][V];
 #pragma unroll
