@@ -159,24 +159,28 @@ __global__ __launch_bounds__(kFinalThreads) void final_backward_kernel(int64_t n
     }
 }
 
-// One wave per column: lane l adds rows l, l + 64, ... in order, then a fixed shuffle tree.
+// One workgroup per column: thread t adds rows t, t + 256, ... in order, a fixed shuffle tree
+// adds the lanes of each wave and the four wave sums are added in order.
 template <typename T>
 __global__ __launch_bounds__(256) void final_reduce_kernel(const T *__restrict__ part, int64_t rows, int64_t nw,
                                                            int64_t ncols, T *__restrict__ gw, T *__restrict__ gb)
 {
-    const int64_t col = (int64_t)blockIdx.x * (256 / kWave) + threadIdx.x / kWave;
-    if (col >= ncols) return;
-    const int l = threadIdx.x % kWave;
+    __shared__ T wave_sum[256 / kWave];
+    const int64_t col = blockIdx.x;
     const T *p = part + col * rows;
     T s = T(0);
-    for (int64_t r = l; r < rows; r += kWave) s += p[r];
+    for (int64_t r = threadIdx.x; r < rows; r += 256) s += p[r];
 #pragma unroll
     for (int off = kWave / 2; off > 0; off >>= 1) s += __shfl_down(s, off, kWave);
-    if (l == 0) {
+    if (threadIdx.x % kWave == 0) wave_sum[threadIdx.x / kWave] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        T total = wave_sum[0];
+        for (int w = 1; w < 256 / kWave; w++) total += wave_sum[w];
         if (col < nw) {
-            if (gw) gw[col] = s;
+            if (gw) gw[col] = total;
         } else if (gb) {
-            gb[col - nw] = s;
+            gb[col - nw] = total;
         }
     }
 }
@@ -264,8 +268,7 @@ hipError_t final_backward(int64_t batch, int c_in, int c_out, int64_t nvox, cons
         o0 += gwd;
     }
     const int64_t nw = (int64_t)c_out * c_in, ncols = nw + c_out;
-    hipLaunchKernelGGL(final_reduce_kernel<T>, dim3((unsigned)((ncols + 3) / 4)), dim3(256), 0, s, ws, rows, nw, ncols,
-                       gw, gb);
+    hipLaunchKernelGGL(final_reduce_kernel<T>, dim3((unsigned)ncols), dim3(256), 0, s, ws, rows, nw, ncols, gw, gb);
     return hipGetLastError();
 }
 
