@@ -25,9 +25,6 @@ const bool g_knobs_ready = [] {
     return true;
 }();
 int knob(Knob k, int dflt) { return g_knobs[k] < 0 ? dflt : g_knobs[k]; }
-// per thread: callers on different threads (one per device under DataParallel) do not meet
-thread_local bool g_reverse_channels = false;
-bool reverse_channels() { return g_reverse_channels; }
 }  // namespace msd
 
 namespace {
@@ -130,6 +127,7 @@ int make_geom(const char *fn, int dtype, int ndim, int64_t batch, int64_t c_in, 
                 return fail(MSD_ERR_INVALID, "%s: Dilation cannot be greater than size of image.", fn);
     }
     g->ndim = ndim;
+    g->reverse = 0;
     g->B = (int)batch;
     g->C = (int)c_in;
     g->Wd = (int)c_out;
@@ -197,11 +195,12 @@ int forward_t(const char *fn, bool relu, const msd::Geom &g, int ndim, const voi
 
 int forward(const char *fn, bool relu, int dtype, int ndim, int64_t batch, int64_t c_in, int64_t c_out,
             const int64_t *spatial, int dilation, const void *input, const int64_t *is, const void *kernel,
-            const void *bias, void *output, const int64_t *os, void *stream)
+            const void *bias, void *output, const int64_t *os, void *stream, bool reverse = false)
 {
     msd::Geom g;
     MSD_TRY(make_geom(fn, dtype, ndim, batch, c_in, c_out, spatial, dilation, true, &g));
     if (c_in <= 0) return fail(MSD_ERR_INVALID, "%s: c_in must be positive", fn);
+    g.reverse = reverse;
     return dtype == MSD_F32
                ? forward_t<float>(fn, relu, g, ndim, input, is, kernel, bias, output, os, (hipStream_t)stream)
                : forward_t<double>(fn, relu, g, ndim, input, is, kernel, bias, output, os, (hipStream_t)stream);
@@ -624,10 +623,9 @@ int block_layer_fused(const char *fn, const BlockArgs &a, int i, int64_t first, 
     MSD_TRY(pending->next(fn, region, &job));
     ProfileScope scope(3, s);
     // as in the forward loop: alternate layers walk the channels in opposite directions
-    msd::g_reverse_channels = msd::knob(msd::kKnobBlockSnake, 1) && (i & 1);
+    g.reverse = msd::knob(msd::kKnobBlockSnake, 1) && (i & 1);
     const hipError_t e = msd::fast_backward_xkb(g, gy, x, (const float *)weights_i, gx, pm, (float *)gk, (float *)gb,
                                                 (float *)ws, s, job);
-    msd::g_reverse_channels = false;
     if (e != hipSuccess) return hip_fail(fn, e);
     if (job) pending->taken(region);
     *done = true;
@@ -667,12 +665,10 @@ int msd_block_forward(int dtype, int ndim, int64_t batch, int64_t c_in, int dept
         // Every second layer walks its input channels from the last to the first: what the
         // layer before touched last is then read first, while it is still in the caches
         // (a few per cent on stacks larger than the 256 MB memory-side cache).
-        msd::g_reverse_channels = msd::knob(msd::kKnobBlockSnake, 1) && (i & 1);
-        const int rc = forward("conv_relu_forward", true, dtype, ndim, batch, first, widths[i], spatial,
-                               (int)dilations[i], stack, stack_strides, weights[i],
-                               (const char *)bias + b0 * a.elem, out, stack_strides, stream);
-        msd::g_reverse_channels = false;
-        MSD_TRY(rc);
+        const bool reverse = msd::knob(msd::kKnobBlockSnake, 1) && (i & 1);
+        MSD_TRY(forward("conv_relu_forward", true, dtype, ndim, batch, first, widths[i], spatial, (int)dilations[i],
+                        stack, stack_strides, weights[i], (const char *)bias + b0 * a.elem, out, stack_strides,
+                        stream, reverse));
         first += widths[i];
         b0 += widths[i];
     }

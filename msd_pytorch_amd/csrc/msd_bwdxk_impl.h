@@ -59,7 +59,6 @@ struct Args {
     RowTeams rt;
     int remap, tiles_per_wg, ngroups, total_groups;
     int group_step;      // 1: a workgroup walks consecutive row groups; > 1: every group_step-th one
-    int reverse;         // walk the blocks of 16 channels from the last to the first
     Plane gy;            // masked output gradient, one channel (sc unused)
     Plane x;             // input channels
     Plane gx;            // grad_input channels (written through a cast)
@@ -162,7 +161,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_rows_fused(const Args a, cons
             }
         };
         // block of 16 channels that stage `s` of the walk belongs to
-        auto block_of = [&](int s) { return a.reverse ? ncb - 1 - s / H : s / H; };
+        auto block_of = [&](int s) { return g.reverse ? ncb - 1 - s / H : s / H; };
         load_stage(block_of(0), 0, ka, ga);   // issued ahead of the gather so the two latencies overlap
 
         // ---- A operands, voxel layout: tv[t][i] = A[t](voxel x0 + i of the team's row)
@@ -441,7 +440,6 @@ hipError_t launch(const Geom &g, const View<const float> &gy, const View<const f
     const int64_t wgs = (total + a.tiles_per_wg - 1) / a.tiles_per_wg;
     const int rows = a.remap ? xcd_grid((int)wgs) : (int)wgs;   // padding workgroups write zero rows
     if (rows > kMaxPartialRows || total > INT32_MAX) return hipErrorInvalidConfiguration;
-    a.reverse = reverse_channels();
     a.group_step = 1;
     if (knob(kKnobBwdkInterleave, 1) && total + rows < INT32_MAX) {
         // the workgroups sweep the image together: at any time they work on one window of

@@ -31,6 +31,8 @@ struct Geom {
     int D, H, W;        // spatial extents (D == 1 in 2D)
     int dil;
     int nvox;           // D * H * W, checked on the host to fit in 31 bits
+    int reverse;        // walk the input channels from the last to the first (same sums, other order);
+                        // set by the dense block's layer loops for every second layer
 };
 
 // Strided view: element strides {batch, channel, z, y, x}.

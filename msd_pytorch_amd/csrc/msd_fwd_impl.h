@@ -38,7 +38,6 @@ struct Lattice {
     int tiles_y;    // dil * segs_y
     int tiles_z;    // dil * segs_z (1 in 2D)
     int ntiles;
-    int reverse;    // walk the input channels from the last to the first
     int by_class;   // 3D: tiles numbered residue class by residue class (2: a class row by row, no blocks)
 };
 
@@ -134,7 +133,7 @@ __global__ __launch_bounds__(1024) void fwd_lattice(Geom g, Lattice lt, int rema
 
     const char *xb = reinterpret_cast<const char *>(x.p + (int64_t)b * x.sb);
     for (int cn = kg; cn < g.C; cn += lt.ks) {
-        const int ci = lt.reverse ? g.C - 1 - cn : cn;
+        const int ci = g.reverse ? g.C - 1 - cn : cn;
         const char *xc = xb + (int64_t)ci * x.sc * 4;
         float w[WOUT][K];
 #pragma unroll
@@ -270,7 +269,6 @@ hipError_t launch(const Geom &g, const View<const float> &x, const float *k, con
 {
     Lattice lt;
     if (!make_lattice(g, V, RZ, RY, knob(kKnobFwdSplit, NDIM == 3 ? 4 : 2), &lt)) return hipErrorInvalidConfiguration;
-    lt.reverse = reverse_channels();
     const int remap = knob(kKnobXcdRemap, 1);
     const dim3 grid(remap ? xcd_grid(lt.ntiles) : lt.ntiles, g.B, 1);
     const size_t lds = (size_t)lt.ks * 3 * V * lt.lpr * sizeof(float);

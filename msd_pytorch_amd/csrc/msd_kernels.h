@@ -54,9 +54,6 @@ enum Knob {
     kKnobCount
 };
 int knob(Knob k, int dflt);
-// Set by the dense block's layer loops: walk the input channels from the last to the first
-// in the next launches (see msd_block_forward).
-bool reverse_channels();
 extern const char *const kKnobNames[kKnobCount];
 extern int g_knobs[kKnobCount];
 
