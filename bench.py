@@ -39,6 +39,7 @@ WORKLOADS = {
     "B": ("regression", 2, 1, 1, 100, 1, 4, (512, 512), True),
     "C": ("segmentation", 2, 1, 4, 100, 1, 1, (1024, 1024), False),
     "D": ("regression", 3, 1, 1, 50, 1, 1, (128, 128, 128), False),
+    "E1": ("regression", 2, 2, 2, 200, 2, 1, (2048, 2048), False),
     "E2": ("regression", 3, 1, 1, 30, 1, 1, (256, 256, 256), False),
 }
 DESCRIPTION = {
@@ -46,6 +47,7 @@ DESCRIPTION = {
     "B": "MSDRegressionModel 2D depth 100 width 1, 4x1x512x512, MSE, fwd+bwd+Adam",
     "C": "MSDSegmentationModel 2D depth 100 width 1 (4 labels), 1x1x1024x1024, NLL, fwd+bwd",
     "D": "MSDRegressionModel 3D depth 50 width 1, 1x1x128x128x128, MSE, fwd+bwd",
+    "E1": "MSDRegressionModel 2D depth 200 width 2, 1x2x2048x2048, MSE, fwd+bwd (13.5 GB of stacks)",
     "E2": "MSDRegressionModel 3D depth 30 width 1, 1x1x256x256x256, MSE, fwd+bwd",
 }
 

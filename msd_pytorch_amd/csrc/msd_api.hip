@@ -530,10 +530,10 @@ int check_block(const char *fn, int dtype, int ndim, int64_t batch, int64_t c_in
 // [0, first) += backward_x, grad_weights/grad_bias += backward_k/bias, the ReLU mask of the
 // layer below applied to its channels on the way out.  *done is false (and nothing was
 // launched) when the fused kernel does not cover the case.
-// Floats of workspace that the partial sums of one fused layer take (one output channel).
-int64_t partial_region_floats(int ndim, int64_t c_in)
+// Floats of workspace that the partial sums of one fused layer take.
+int64_t partial_region_floats(int ndim, int64_t c_in, int64_t width)
 {
-    return (c_in * (ndim == 3 ? 27 : 9) + 1) * (int64_t)msd::kMaxPartialRows;
+    return width * (c_in * (ndim == 3 ? 27 : 9) + 1) * (int64_t)msd::kMaxPartialRows;
 }
 
 constexpr int64_t kDeferBudgetBytes = (int64_t)1 << 30;   // most workspace spent on pending partial sums
@@ -618,7 +618,7 @@ int block_layer_fused(const char *fn, const BlockArgs &a, int i, int64_t first, 
             *masked = true;
         }
     }
-    const int64_t region = partial_region_floats(a.ndim, g.C);
+    const int64_t region = partial_region_floats(a.ndim, g.C, g.Wd);
     msd::ReduceJob *job = nullptr;
     MSD_TRY(pending->next(fn, region, &job));
     ProfileScope scope(3, s);
@@ -644,7 +644,8 @@ int64_t msd_block_workspace_bytes(int dtype, int ndim, int64_t batch, int64_t c_
     // their reductions can wait for one another
     int64_t regions = 0, total = c_in;
     for (int i = 0; i < depth; i++) {
-        if (dtype == MSD_F32 && widths[i] == 1) regions += partial_region_floats(ndim, total) * (int64_t)sizeof(float);
+        if (dtype == MSD_F32 && widths[i] <= 2)
+            regions += partial_region_floats(ndim, total, widths[i]) * (int64_t)sizeof(float);
         total += widths[i];
     }
     return need + (regions < kDeferBudgetBytes ? regions : kDeferBudgetBytes);

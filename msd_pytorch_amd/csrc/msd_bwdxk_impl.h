@@ -42,10 +42,11 @@ using bwdk::kThreads;
 using bwdk::kWaves;
 using bwdk::mfma4;
 
-// Wave-private LDS tile [tap][voxel]; one more row of zeros feeds the MFMA rows past K.
-template <int NDIM, int V> struct ATile {
+// Wave-private LDS tile [output channel][tap][voxel]; one more row of zeros feeds the MFMA
+// rows past the last tap.
+template <int NDIM, int V, int WOUT> struct ATile {
     static constexpr int kStride = kWave * V + 4;     // floats per row (bank spread for the b128 reads)
-    static constexpr int kRows = Taps<NDIM>::K + 1;
+    static constexpr int kRows = WOUT * Taps<NDIM>::K + 1;
     static constexpr int kFloats = kRows * kStride;
 };
 
@@ -59,14 +60,14 @@ struct Args {
     RowTeams rt;
     int remap, tiles_per_wg, ngroups, total_groups;
     int group_step;      // 1: a workgroup walks consecutive row groups; > 1: every group_step-th one
-    Plane gy;            // masked output gradient, one channel (sc unused)
+    Plane gy;            // masked output gradient, one or two channels
     Plane x;             // input channels
     Plane gx;            // grad_input channels (written through a cast)
     int mask_from;       // activations (viewed like grad_input) mask the channels >= mask_from
     int want_bias;
 };
 
-template <int NDIM, int V, int NCB>
+template <int NDIM, int V, int NCB, int WOUT>
 __global__ __launch_bounds__(kThreads, 2) void bwd_rows_fused(const Args a, const float *__restrict__ gyp,
                                                               const float *__restrict__ xp, float *__restrict__ gxp,
                                                               const float *__restrict__ actp,
@@ -76,11 +77,12 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_rows_fused(const Args a, cons
     // are then known not to change under the stores to grad_input and stay scalar loads
     extern __shared__ float lds[];
     constexpr int K = Taps<NDIM>::K, NPQ = RowTaps<NDIM>::NPQ;
-    constexpr int TG = NDIM == 3 ? 2 : 1;         // groups of 16 tap rows
+    constexpr int KR = WOUT * K;                  // rows of the A tile: (output channel, tap)
+    constexpr int TG = (KR + 15) / 16;            // groups of 16 such rows
     constexpr int NSS = V == 1 ? 2 : 4;           // 16-voxel MFMA groups per pipeline stage
     constexpr int H = 4 * V / NSS;                // stages per block of 16 channels (even)
     constexpr int NCS = kChanBlock / H;           // grad_input channels per stage
-    constexpr int ASTRIDE = ATile<NDIM, V>::kStride;
+    constexpr int ASTRIDE = ATile<NDIM, V, WOUT>::kStride;
     const Geom &g = a.g;
     const RowTeams &rt = a.rt;
     const int tid = threadIdx.x;
@@ -88,9 +90,9 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_rows_fused(const Args a, cons
     const int wave = __builtin_amdgcn_readfirstlane(tid / kWave), wl = tid % kWave;
     const int mk = wl / 16, mj = wl % 16;         // MFMA k (voxel group) and i/j (tap or channel) of this lane
     const int team = tid / rt.lpr, lane = tid % rt.lpr;
-    float *S = lds + (size_t)team * NPQ * V * rt.lpr;
-    float *AT = lds + (size_t)rt.rpw * NPQ * V * rt.lpr + (size_t)wave * ATile<NDIM, V>::kFloats;
-    for (int i = wl; i < ASTRIDE; i += kWave) AT[K * ASTRIDE + i] = 0.f;
+    float *S = lds + (size_t)team * WOUT * NPQ * V * rt.lpr;
+    float *AT = lds + (size_t)rt.rpw * WOUT * NPQ * V * rt.lpr + (size_t)wave * ATile<NDIM, V, WOUT>::kFloats;
+    for (int i = wl; i < ASTRIDE; i += kWave) AT[KR * ASTRIDE + i] = 0.f;
 
     const int c0 = blockIdx.z * NCB * kChanBlock;
     const int ones_ch = a.want_bias ? g.C : -1;   // virtual channel of ones -> bias sum
@@ -110,7 +112,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_rows_fused(const Args a, cons
     const int kx = (lane - wl) * V + 4 * mk;      // first voxel of this lane's MFMA groups, + 16 s
     int arow[TG];                                 // this lane's row of the A tile (the zero row past K taps)
 #pragma unroll
-    for (int tg = 0; tg < TG; tg++) arow[tg] = min(tg * 16 + mj, K) * ASTRIDE + 4 * mk;
+    for (int tg = 0; tg < TG; tg++) arow[tg] = min(tg * 16 + mj, KR) * ASTRIDE + 4 * mk;
 
     // Position of the lane's row, advanced from tile to tile without divisions: the row groups
     // of a workgroup are consecutive.
@@ -164,20 +166,20 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_rows_fused(const Args a, cons
         auto block_of = [&](int s) { return g.reverse ? ncb - 1 - s / H : s / H; };
         load_stage(block_of(0), 0, ka, ga);   // issued ahead of the gather so the two latencies overlap
 
-        // ---- A operands, voxel layout: tv[t][i] = A[t](voxel x0 + i of the team's row)
-        float tv[K][V];
+        // ---- A operands, voxel layout: tv[co * K + t][i] = A_co[t](voxel x0 + i of the team's row)
+        float tv[KR][V];
         {
             const View<const float> none{nullptr, 0, 0, 0, 0, 0};
-            const View<const float> gyv{gyp, a.gy.sb, 0, a.gy.sz, a.gy.sy, 1};
-            float own[1][NPQ][V];
-            stage_source_rows<NDIM, false, 1, V>(g, rt, none, gyv, b, zc, yc, lane, act, S, own);
+            const View<const float> gyv{gyp, a.gy.sb, a.gy.sc, a.gy.sz, a.gy.sy, 1};
+            float own[WOUT][NPQ][V];
+            stage_source_rows<NDIM, false, WOUT, V>(g, rt, none, gyv, b, zc, yc, lane, act, S, own);
             // per voxel: all LDS reads first, so that their latencies overlap, then the sums
 #pragma unroll
             for (int i = 0; i < V; i++) {
                 const SideTaps<V> side(min(x0 + i, g.W - 1), g.W, g.dil, rt.lpr);
-                float ra[NPQ][4];
+                float ra[WOUT * NPQ][4];
 #pragma unroll
-                for (int pq = 0; pq < NPQ; pq++) {
+                for (int pq = 0; pq < WOUT * NPQ; pq++) {
                     const float *srow = S + (size_t)pq * V * rt.lpr;
                     ra[pq][0] = srow[side.i0a];
                     ra[pq][1] = srow[side.i0b];
@@ -186,17 +188,20 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_rows_fused(const Args a, cons
                 }
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int pq = 0; pq < NPQ; pq++) {
-                    tv[pq * 3 + 0][i] = (side.m0a ? ra[pq][0] : 0.f) + (side.m0b ? ra[pq][1] : 0.f);
-                    tv[pq * 3 + 1][i] = own[0][pq][i];
-                    tv[pq * 3 + 2][i] = (side.m2a ? ra[pq][2] : 0.f) + (side.m2b ? ra[pq][3] : 0.f);
-                }
+                for (int co = 0; co < WOUT; co++)
+#pragma unroll
+                    for (int pq = 0; pq < NPQ; pq++) {
+                        const int r = co * NPQ + pq;   // staged row; its three taps are rows 3 r .. 3 r + 2 of tv
+                        tv[r * 3 + 0][i] = (side.m0a ? ra[r][0] : 0.f) + (side.m0b ? ra[r][1] : 0.f);
+                        tv[r * 3 + 1][i] = own[co][pq][i];
+                        tv[r * 3 + 2][i] = (side.m2a ? ra[r][2] : 0.f) + (side.m2b ? ra[r][3] : 0.f);
+                    }
                 __builtin_amdgcn_sched_barrier(0);
             }
             __syncthreads();                      // the staged rows may be overwritten from here on
-            // the wave's [tap][voxel] tile; lanes past the row hold finite values that meet zeros of x
+            // the wave's [row][voxel] tile; lanes past the image row hold finite values that meet zeros of x
 #pragma unroll
-            for (int t = 0; t < K; t++) store_vec<V>(AT + t * ASTRIDE + wl * V, tv[t]);
+            for (int t = 0; t < KR; t++) store_vec<V>(AT + t * ASTRIDE + wl * V, tv[t]);
         }
         // the tile is private to the wave and LDS executes a wave's accesses in order: only
         // the compiler has to be kept from reordering them
@@ -227,17 +232,20 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_rows_fused(const Args a, cons
                 }
             }
         };
-        // grad_input of one channel: K * V fused multiply-adds with the channel's weights
+        // grad_input of one channel: WOUT * K * V fused multiply-adds with the channel's weights
         // (wave-uniform: scalar loads into scalar registers), then the store
-        auto load_weights = [&](int ci, float (&w)[K]) {
-            const float *kc = kw + (int64_t)ci * K;
+        auto load_weights = [&](int ci, float (&w)[KR]) {
 #pragma unroll
-            for (int t = 0; t < K; t++) w[t] = kc[t];
+            for (int co = 0; co < WOUT; co++) {
+                const float *kc = kw + ((int64_t)co * g.C + ci) * K;
+#pragma unroll
+                for (int t = 0; t < K; t++) w[co * K + t] = kc[t];
+            }
         };
         // `prefetch`: the weights of the next channel are requested right after the first use
         // of this channel's (scalar loads return in any order, so only a wait for all of them
         // exists: the request must follow that wait to have the rest of the arithmetic to land in)
-        auto update_channel = [&](int ci, float (&gv)[V], const float (&w)[K], auto prefetch, float (&wn)[K],
+        auto update_channel = [&](int ci, float (&gv)[V], const float (&w)[KR], auto prefetch, float (&wn)[KR],
                                   bool masked) {
             float sum[V];
 #pragma unroll
@@ -246,7 +254,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_rows_fused(const Args a, cons
             if (decltype(prefetch)::value) load_weights(ci + 1, wn);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int t = 1; t < K; t++)
+            for (int t = 1; t < KR; t++)
 #pragma unroll
                 for (int i = 0; i < V; i++) sum[i] += w[t] * tv[t][i];
 #pragma unroll
@@ -268,7 +276,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_rows_fused(const Args a, cons
             const int cj0 = c0 + cb * kChanBlock + h * NCS;
             if (!act) return;
             asm volatile("" : "+v"(goff));        // as in load_stage: the stores take base + lane offset directly
-            float w[2][K];
+            float w[2][KR];
             if (cj0 + NCS <= min(cx_end, a.mask_from)) {   // uniform
                 load_weights(cj0, w[0]);
 #pragma unroll
@@ -367,24 +375,25 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_rows_fused(const Args a, cons
     float *pcol = part + blockIdx.x;
     for (int idx = tid; idx < PER_WAVE; idx += blockDim.x) {
         const int l = idx % kWave, v = (idx / kWave) % 4, tg = (idx / (4 * kWave)) % TG, cb = idx / (4 * kWave * TG);
-        const int tap = tg * 16 + 4 * (l / 16) + v;
+        const int r = tg * 16 + 4 * (l / 16) + v;     // row of the A tile: (output channel, tap)
         const int ch = c0 + cb * kChanBlock + l % 16;
-        if (tap >= K || ch >= c_end) continue;
+        if (r >= KR || ch >= c_end) continue;
+        const int co = r / K, tap = r % K;
         float s = 0.f;
         for (int w = 0; w < nwaves; w++) s += red[w * PER_WAVE + idx];
         if (ch < g.C)
-            pcol[((int64_t)ch * K + tap) * kMaxPartialRows] = s;
+            pcol[(((int64_t)co * g.C + ch) * K + tap) * kMaxPartialRows] = s;
         else if (tap == K / 2)
-            pcol[((int64_t)g.C * K) * kMaxPartialRows] = s;
+            pcol[((int64_t)WOUT * g.C * K + co) * kMaxPartialRows] = s;
     }
 }
 
-template <int NDIM, int V, int NCB>
+template <int NDIM, int V, int NCB, int WOUT>
 size_t lds_bytes(const RowTeams &rt)
 {
-    constexpr int TG = NDIM == 3 ? 2 : 1;
-    const size_t main_loop =
-        ((size_t)rt.rpw * RowTaps<NDIM>::NPQ * V * rt.lpr + (size_t)kWaves * ATile<NDIM, V>::kFloats) * 4;
+    constexpr int TG = (WOUT * Taps<NDIM>::K + 15) / 16;
+    const size_t main_loop = ((size_t)rt.rpw * WOUT * RowTaps<NDIM>::NPQ * V * rt.lpr +
+                              (size_t)kWaves * ATile<NDIM, V, WOUT>::kFloats) * 4;
     const size_t epilogue = (size_t)kWaves * NCB * TG * 4 * kWave * 4;
     return std::max(main_loop, epilogue);
 }
@@ -420,7 +429,7 @@ int choose_vec(const Geom &g, int vmax, const View<const float> &gy, const View<
     return 0;
 }
 
-template <int NDIM, int V, int NCB>
+template <int NDIM, int V, int NCB, int WOUT>
 hipError_t launch(const Geom &g, const View<const float> &gy, const View<const float> &x, const float *k,
                   const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws, hipStream_t s,
                   ReduceJob *defer)
@@ -455,13 +464,13 @@ hipError_t launch(const Geom &g, const View<const float> &gy, const View<const f
     a.mask_from = pm.from;
     a.want_bias = gb != nullptr;
     const int chunks = (g.C + a.want_bias + NCB * kChanBlock - 1) / (NCB * kChanBlock);
-    const size_t lds = lds_bytes<NDIM, V, NCB>(a.rt);
-    hipLaunchKernelGGL((bwd_rows_fused<NDIM, V, NCB>), dim3(rows, 1, chunks), dim3(a.rt.lpr * a.rt.rpw), lds, s, a,
+    const size_t lds = lds_bytes<NDIM, V, NCB, WOUT>(a.rt);
+    hipLaunchKernelGGL((bwd_rows_fused<NDIM, V, NCB, WOUT>), dim3(rows, 1, chunks), dim3(a.rt.lpr * a.rt.rpw), lds, s, a,
                        gy.p, x.p, gx.p, actp, k, part);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    const int64_t nk = (int64_t)g.C * K;
-    const int64_t ncols = nk + (a.want_bias ? 1 : 0);
+    const int64_t nk = (int64_t)WOUT * g.C * K;
+    const int64_t ncols = nk + (a.want_bias ? WOUT : 0);
     if (defer) {
         *defer = ReduceJob{part, gk, gb, nk, ncols, rows};
         return hipSuccess;
@@ -470,23 +479,34 @@ hipError_t launch(const Geom &g, const View<const float> &gy, const View<const f
     return hipGetLastError();
 }
 
-template <int NDIM, int V>
+template <int NDIM, int V, int WOUT>
 hipError_t pick_ncb(const Geom &g, const View<const float> &gy, const View<const float> &x, const float *k,
                     const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws, hipStream_t s,
                     ReduceJob *defer)
 {
     const int need = (g.C + (gb != nullptr) + kChanBlock - 1) / kChanBlock;
-    if (need <= 1) return launch<NDIM, V, 1>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
-    if (need <= 2) return launch<NDIM, V, 2>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
-    if (need <= 4) return launch<NDIM, V, 4>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
-    return launch<NDIM, V, 8>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
+    if (need <= 1) return launch<NDIM, V, 1, WOUT>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
+    if (need <= 2) return launch<NDIM, V, 2, WOUT>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
+    if (need <= 4) return launch<NDIM, V, 4, WOUT>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
+    return launch<NDIM, V, 8, WOUT>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
 }
 
-// One output channel, unit x-strides, 32-bit strides, and a vector width that fits.
+// Widest vector for two output channels (2D only): twice the gathered values per voxel must
+// still fit the registers beside the pipeline buffers.
+constexpr int kMaxVecTwoOutputs = 2;
+
+// One output channel (2D: one or two), unit x-strides, 32-bit strides, and a vector width
+// that fits.
 template <int NDIM>
 bool xkb_supported_nd(const Geom &g, const View<const float> &gy, const View<const float> &x, const View<float> &gx)
 {
-    if (g.Wd != 1 || x.sx != 1 || gy.sx != 1 || gx.sx != 1) return false;
+    if (g.Wd != 1 && !(NDIM == 2 && g.Wd == 2)) return false;
+    if (x.sx != 1 || gy.sx != 1 || gx.sx != 1) return false;
+    if (g.Wd == 2) {
+        if (!small_strides(g, gy) || !small_strides(g, x) || !small_strides(g, gx)) return false;
+        if ((int64_t)g.C * x.sc + (int64_t)g.D * x.sz + (int64_t)g.H * x.sy + g.W >= ((int64_t)1 << 30)) return false;
+        return choose_vec<NDIM>(g, kMaxVecTwoOutputs, gy, x, gx) != 0;
+    }
     if (!small_strides(g, gy) || !small_strides(g, x) || !small_strides(g, gx)) return false;
     if ((int64_t)g.C * x.sc + (int64_t)g.D * x.sz + (int64_t)g.H * x.sy + g.W >= ((int64_t)1 << 30)) return false;
     return choose_vec<NDIM>(g, 4, gy, x, gx) != 0;
@@ -503,10 +523,18 @@ hipError_t xkb_nd(const Geom &g, const View<const float> &gy, const View<const f
     int v = choose_vec<NDIM>(g, vmax, gy, x, gx);
     if (v == 0) v = choose_vec<NDIM>(g, 4, gy, x, gx);
     if constexpr (NDIM == 2) {
-        if (v == 4) return pick_ncb<2, 4>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
+        if (g.Wd == 2) {
+            v = choose_vec<2>(g, std::min(vmax, kMaxVecTwoOutputs), gy, x, gx);
+            if (v == 0) v = choose_vec<2>(g, kMaxVecTwoOutputs, gy, x, gx);
+            if (v == 2) return pick_ncb<2, 2, 2>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
+            if (v == 1) return pick_ncb<2, 1, 2>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
+            return hipErrorInvalidConfiguration;
+        }
+        if (v == 4) return pick_ncb<2, 4, 1>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
     }
-    if (v == 2) return pick_ncb<NDIM, 2>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
-    if (v == 1) return pick_ncb<NDIM, 1>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
+    if (g.Wd != 1) return hipErrorInvalidConfiguration;
+    if (v == 2) return pick_ncb<NDIM, 2, 1>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
+    if (v == 1) return pick_ncb<NDIM, 1, 1>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
     return hipErrorInvalidConfiguration;
 }
 

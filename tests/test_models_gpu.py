@@ -55,7 +55,7 @@ def test_block_matches_oracle(ndim, size, c_in, width, depth, dtype):
         assert rel_err(a.grad, b) <= tg
 
 
-@pytest.mark.parametrize("ndim,size,c_in,depth,batch,dilations", [
+FUSED_BLOCK_CASES = [
     # shapes the fused backward_x + backward_k kernel of the block takes (width 1, rows of
     # whole 4-voxel groups and at least one wavefront), with ragged rows, row groups and
     # channel blocks (16 input channels each, plus the bias column)
@@ -68,11 +68,17 @@ def test_block_matches_oracle(ndim, size, c_in, width, depth, dtype):
     (3, (12, 5, 64), 1, 3, 1, [5, 1, 4]),  # dilation == smallest extent
     (2, (700, 260), 1, 3, 2, None),        # more row groups than workgroups: several tiles each
     (3, (33, 31, 68), 2, 3, 2, None),      # the same in 3D, last groups ragged
-])
-def test_fused_block_backward_matches_oracle(ndim, size, c_in, depth, batch, dilations):
+    (2, (21, 128), 2, 11, 1, None, 2),     # width 2: two output channels per layer in the fused pass
+    (2, (300, 132), 2, 4, 2, None, 2),     # width 2, several tiles per workgroup
+]
+
+
+@pytest.mark.parametrize("ndim,size,c_in,depth,batch,dilations,width",
+                         [c if len(c) == 7 else c + (1,) for c in FUSED_BLOCK_CASES])
+def test_fused_block_backward_matches_oracle(ndim, size, c_in, depth, batch, dilations, width):
     from msd_pytorch_amd import _native
     from msd_pytorch_amd.msd_block import msd_block
-    x, dil, bias, ws, g = make_block_problem(ndim, size, c_in, 1, depth, torch.float32, batch=batch)
+    x, dil, bias, ws, g = make_block_problem(ndim, size, c_in, width, depth, torch.float32, batch=batch)
     if dilations is not None:
         dil = dilations
     want = oracle.block_forward(x.double(), dil, bias.double(), [w.double() for w in ws])

@@ -171,6 +171,9 @@ SHAPES_XKB = [
     (2, 3, 1, (9, 1024), 9),          # one row per workgroup, dilation == height
     (1, 40, 1, (6, 7, 128), 3),       # 3D, 3 channel blocks
     (1, 2, 1, (4, 5, 68), 4),         # 3D, ragged row
+    (2, 5, 2, (7, 128), 2),           # two output channels: 2 voxels per lane, 2 rows per workgroup
+    (1, 35, 2, (12, 512), 5),         # two output channels, 3 channel blocks, one row per workgroup
+    (1, 16, 2, (9, 68), 3),           # two output channels, one voxel per lane, bias column in a block of its own
 ]
 
 
@@ -179,7 +182,7 @@ SHAPES_XKB = [
                                                 SHAPES_FAST[5], SHAPES_FAST[6], SHAPES_FAST[9]])
 def test_backward_xkb_equals_the_three_operators(cc, shape, dtype):
     # one call (one pass over the channels where the fused kernel applies; fp64, two output
-    # channels and odd row lengths take the separate kernels) against the oracle's
+    # channels in 3D and odd row lengths take the separate kernels) against the oracle's
     # conv_backward_x, conv_backward_k and conv_backward_bias, all accumulating
     ref = make_problem(shape, dtype, seed=5)
     dev = make_problem(shape, dtype, device="cuda", seed=5)
