@@ -42,7 +42,7 @@ struct Lattice {
 };
 
 template <int NDIM, bool RELU, int WOUT, int V, int RZ, int RY>
-__global__ __launch_bounds__(1024) void fwd_lattice(Geom g, Lattice lt, int remap, View<const float> x,
+__global__ __launch_bounds__(NDIM == 3 ? 512 : 1024, (NDIM == 3 && V == 1 && WOUT == 1) ? 8 : 1) void fwd_lattice(Geom g, Lattice lt, int remap, View<const float> x,
                                                     const float *__restrict__ k, const float *__restrict__ bias,
                                                     View<float> out)
 {
