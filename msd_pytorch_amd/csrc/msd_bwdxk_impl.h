@@ -95,10 +95,17 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_rows_fused(const Args a, cons
     for (int i = wl; i < ASTRIDE; i += kWave) AT[KR * ASTRIDE + i] = 0.f;
 
     const int c0 = blockIdx.z * NCB * kChanBlock;
-    const int ones_ch = a.want_bias ? g.C : -1;   // virtual channel of ones -> bias sum
-    const int c_end = min(g.C + (a.want_bias ? 1 : 0), c0 + NCB * kChanBlock);
-    const int cx_end = min(c_end, g.C);           // real channels of this chunk end here
+    const int c_end = min(g.C, c0 + NCB * kChanBlock);   // channels of this chunk end here
+    const int cx_end = c_end;
     const int ncb = (c_end - c0 + kChanBlock - 1) / kChanBlock;
+    // The bias gradient is the sum of the centre tap over all voxels: every lane adds up its
+    // own voxels (chunk 0 only) and the workgroup reduces them at the end.  A virtual input
+    // channel of ones on the matrix cores would do it too, but costs a whole block of 16
+    // channels more whenever C is a multiple of 16.
+    const bool sum_bias = a.want_bias && blockIdx.z == 0;
+    float bsum[WOUT];
+#pragma unroll
+    for (int co = 0; co < WOUT; co++) bsum[co] = 0.f;
 
     mfma4 D[NCB][TG];
 #pragma unroll
@@ -202,6 +209,12 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_rows_fused(const Args a, cons
             // the wave's [row][voxel] tile; lanes past the image row hold finite values that meet zeros of x
 #pragma unroll
             for (int t = 0; t < KR; t++) store_vec<V>(AT + t * ASTRIDE + wl * V, tv[t]);
+            if (sum_bias && act) {
+#pragma unroll
+                for (int co = 0; co < WOUT; co++)
+#pragma unroll
+                    for (int i = 0; i < V; i++) bsum[co] += tv[co * K + K / 2][i];
+            }
         }
         // the tile is private to the wave and LDS executes a wave's accesses in order: only
         // the compiler has to be kept from reordering them
@@ -213,19 +226,18 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_rows_fused(const Args a, cons
         // weight gradient of one stage: 4 * NSS * TG matrix instructions
         auto stage_k = [&](int cb, int h, float (&kk)[NSS][4]) {
             const int chl = c0 + cb * kChanBlock + mj;
-            const bool chok = chl < g.C, one = chl == ones_ch;
+            const bool chok = chl < g.C;
 #pragma unroll
             for (int j = 0; j < NSS; j++) {
                 const int s = h * NSS + j;
                 const bool vok = rowok && kx + 16 * s < g.W;
                 const bool keep = vok && chok;
-                const float fill = (vok && one) ? 1.f : 0.f;
                 f32x4 av[TG];
 #pragma unroll
                 for (int tg = 0; tg < TG; tg++) av[tg] = *reinterpret_cast<const f32x4 *>(AT + arow[tg] + 16 * s);
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    const float bv = keep ? kk[j][e] : fill;
+                    const float bv = keep ? kk[j][e] : 0.f;
 #pragma unroll
                     for (int tg = 0; tg < TG; tg++)
                         acc[tg][e & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[tg][e], bv, acc[tg][e & 1], 0, 0, 0);
@@ -381,10 +393,24 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_rows_fused(const Args a, cons
         const int co = r / K, tap = r % K;
         float s = 0.f;
         for (int w = 0; w < nwaves; w++) s += red[w * PER_WAVE + idx];
-        if (ch < g.C)
-            pcol[(((int64_t)co * g.C + ch) * K + tap) * kMaxPartialRows] = s;
-        else if (tap == K / 2)
-            pcol[((int64_t)WOUT * g.C * K + co) * kMaxPartialRows] = s;
+        pcol[(((int64_t)co * g.C + ch) * K + tap) * kMaxPartialRows] = s;
+    }
+    if (sum_bias) {                               // uniform over the workgroup
+        // lanes of a wave by a fixed shuffle tree, then the waves in order
+        __syncthreads();
+#pragma unroll
+        for (int co = 0; co < WOUT; co++) {
+            float s = bsum[co];
+#pragma unroll
+            for (int off = kWave / 2; off > 0; off >>= 1) s += __shfl_down(s, off, kWave);
+            if (wl == 0) red[wave * WOUT + co] = s;
+        }
+        __syncthreads();
+        if (tid < WOUT) {
+            float s = 0.f;
+            for (int w = 0; w < nwaves; w++) s += red[w * WOUT + tid];
+            pcol[((int64_t)WOUT * g.C * K + tid) * kMaxPartialRows] = s;
+        }
     }
 }
 
@@ -463,7 +489,7 @@ hipError_t launch(const Geom &g, const View<const float> &gy, const View<const f
     const float *actp = pm.from < g.C ? pm.act.p : x.p;   // only dereferenced for channels >= mask_from
     a.mask_from = pm.from;
     a.want_bias = gb != nullptr;
-    const int chunks = (g.C + a.want_bias + NCB * kChanBlock - 1) / (NCB * kChanBlock);
+    const int chunks = (g.C + NCB * kChanBlock - 1) / (NCB * kChanBlock);
     const size_t lds = lds_bytes<NDIM, V, NCB, WOUT>(a.rt);
     hipLaunchKernelGGL((bwd_rows_fused<NDIM, V, NCB, WOUT>), dim3(rows, 1, chunks), dim3(a.rt.lpr * a.rt.rpw), lds, s, a,
                        gy.p, x.p, gx.p, actp, k, part);
@@ -484,7 +510,7 @@ hipError_t pick_ncb(const Geom &g, const View<const float> &gy, const View<const
                     const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws, hipStream_t s,
                     ReduceJob *defer)
 {
-    const int need = (g.C + (gb != nullptr) + kChanBlock - 1) / kChanBlock;
+    const int need = (g.C + kChanBlock - 1) / kChanBlock;
     if (need <= 1) return launch<NDIM, V, 1, WOUT>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
     if (need <= 2) return launch<NDIM, V, 2, WOUT>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
     if (need <= 4) return launch<NDIM, V, 4, WOUT>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);

@@ -58,7 +58,7 @@ def test_block_matches_oracle(ndim, size, c_in, width, depth, dtype):
 FUSED_BLOCK_CASES = [
     # shapes the fused backward_x + backward_k kernel of the block takes (width 1, rows of
     # whole 4-voxel groups and at least one wavefront), with ragged rows, row groups and
-    # channel blocks (16 input channels each, plus the bias column)
+    # channel blocks (16 input channels each)
     (2, (37, 256), 1, 20, 2, None),        # 4 voxels per lane, 4 rows per workgroup, 37 rows
     (2, (9, 1024), 2, 5, 1, None),         # one row per workgroup
     (2, (30, 132), 3, 36, 1, None),        # 33 of 64 lanes per row busy; 3 channel blocks

@@ -167,13 +167,13 @@ def test_mask_once_then_plain_operators(cc, shape, dtype):
 # shapes the one-pass kernel behind conv_backward_xkb takes (one output channel, rows of whole
 # 4-voxel groups, at least one wavefront per row), beside the SHAPES_FAST ones that qualify
 SHAPES_XKB = [
-    (1, 17, 1, (5, 256), 2),          # 4 voxels per lane, 4 rows per workgroup, 2 channel blocks with the bias
+    (1, 17, 1, (5, 256), 2),          # 4 voxels per lane, 4 rows per workgroup, 2 channel blocks
     (2, 3, 1, (9, 1024), 9),          # one row per workgroup, dilation == height
     (1, 40, 1, (6, 7, 128), 3),       # 3D, 3 channel blocks
     (1, 2, 1, (4, 5, 68), 4),         # 3D, ragged row
     (2, 5, 2, (7, 128), 2),           # two output channels: 2 voxels per lane, 2 rows per workgroup
     (1, 35, 2, (12, 512), 5),         # two output channels, 3 channel blocks, one row per workgroup
-    (1, 16, 2, (9, 68), 3),           # two output channels, one voxel per lane, bias column in a block of its own
+    (1, 16, 2, (9, 68), 3),           # two output channels, one voxel per lane, exactly one channel block
 ]
 
 
