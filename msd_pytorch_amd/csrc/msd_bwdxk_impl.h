@@ -67,11 +67,19 @@ struct Args {
     int want_bias;
 };
 
+// Workgroups (of four waves) that are resident per CU: the 3D kernel with one voxel per lane
+// and at most 32 channels per chunk fits 168 registers, so three of them share a CU; the
+// others need up to 256 registers, which leaves room for two.
+template <int NDIM, int V, int NCB, int WOUT> constexpr int resident_per_cu()
+{
+    return (NDIM == 3 && V == 1 && WOUT == 1 && NCB <= 2) ? 3 : 2;
+}
+
 template <int NDIM, int V, int NCB, int WOUT>
-__global__ __launch_bounds__(kThreads, 2) void bwd_rows_fused(const Args a, const float *__restrict__ gyp,
-                                                              const float *__restrict__ xp, float *__restrict__ gxp,
-                                                              const float *__restrict__ actp,
-                                                              const float *__restrict__ kw, float *__restrict__ part)
+__global__ __launch_bounds__(kThreads, (resident_per_cu<NDIM, V, NCB, WOUT>()))
+void bwd_rows_fused(const Args a, const float *__restrict__ gyp, const float *__restrict__ xp,
+                    float *__restrict__ gxp, const float *__restrict__ actp, const float *__restrict__ kw,
+                    float *__restrict__ part)
 {
     // the pointers are separate arguments so that they can carry __restrict__: the weights
     // are then known not to change under the stores to grad_input and stay scalar loads
@@ -469,8 +477,9 @@ hipError_t launch(const Geom &g, const View<const float> &gy, const View<const f
     a.ngroups = (a.rt.nrows + a.rt.rpw - 1) / a.rt.rpw;
     const int64_t total = (int64_t)a.ngroups * g.B;
     a.remap = knob(kKnobXcdRemap, 1);
-    // two workgroups per CU are resident (registers): with that many the grid runs as one round
-    const int64_t max_wgs = std::min<int64_t>(std::max(8, knob(kKnobBwdkBlocks, 512)), kMaxPartialRows);
+    // as many workgroups as are resident at once (256 CUs): the grid then runs as one round
+    const int64_t max_wgs = std::min<int64_t>(
+        std::max(8, knob(kKnobBwdkBlocks, 256 * resident_per_cu<NDIM, V, NCB, WOUT>())), kMaxPartialRows);
     a.tiles_per_wg = (int)((total + max_wgs - 1) / max_wgs);
     const int64_t wgs = (total + a.tiles_per_wg - 1) / a.tiles_per_wg;
     const int rows = a.remap ? xcd_grid((int)wgs) : (int)wgs;   // padding workgroups write zero rows
