@@ -29,8 +29,8 @@ HBM_PEAK_GBS = 8000.0
 # WRITE_SIZE x 1.000).  Counters cannot be read from inside this script, so the figures
 # of the committed profiles are carried here; a class without one reports null.
 TRAFFIC = {
-    "C": {"forward": 22.213e9, "backward_xkb": 65.910e9 + 0.096e9},
-    "D": {"forward": 15.318e9, "backward_xkb": 34.009e9 + 0.072e9},
+    "C": {"forward": 22.210e9, "backward_xkb": 65.896e9 + 0.096e9},
+    "D": {"forward": 16.187e9, "backward_xkb": 34.848e9 + 0.072e9},
 }
 
 WORKLOADS = {
