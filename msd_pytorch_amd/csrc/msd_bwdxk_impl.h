@@ -68,11 +68,12 @@ struct Args {
 };
 
 // Workgroups (of four waves) that are resident per CU: the 3D kernel with one voxel per lane
-// and at most 32 channels per chunk fits 168 registers, so three of them share a CU; the
-// others need up to 256 registers, which leaves room for two.
+// and at most 64 channels per chunk fits 168 registers (the 64-channel one with pipeline
+// stages of 16 voxels instead of 32), so three of them share a CU; the others need up to
+// 256 registers, which leaves room for two.
 template <int NDIM, int V, int NCB, int WOUT> constexpr int resident_per_cu()
 {
-    return (NDIM == 3 && V == 1 && WOUT == 1 && NCB <= 2) ? 3 : 2;
+    return (NDIM == 3 && V == 1 && WOUT == 1 && NCB <= 4) ? 3 : 2;
 }
 
 template <int NDIM, int V, int NCB, int WOUT>
@@ -87,7 +88,7 @@ void bwd_rows_fused(const Args a, const float *__restrict__ gyp, const float *__
     constexpr int K = Taps<NDIM>::K, NPQ = RowTaps<NDIM>::NPQ;
     constexpr int KR = WOUT * K;                  // rows of the A tile: (output channel, tap)
     constexpr int TG = (KR + 15) / 16;            // groups of 16 such rows
-    constexpr int NSS = V == 1 ? 2 : 4;           // 16-voxel MFMA groups per pipeline stage
+    constexpr int NSS = V == 1 ? (NCB == 4 ? 1 : 2) : 4;   // 16-voxel MFMA groups per pipeline stage
     constexpr int H = 4 * V / NSS;                // stages per block of 16 channels (even)
     constexpr int NCS = kChanBlock / H;           // grad_input channels per stage
     constexpr int ASTRIDE = ATile<NDIM, V, WOUT>::kStride;
