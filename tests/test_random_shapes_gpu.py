@@ -1,0 +1,124 @@
+"""Seeded random problems against the CPU oracle: operators and whole blocks at shapes nobody
+picked by hand (ragged rows, row lengths around the kernels' limits, dilations up to the
+smallest extent, one or two output channels, batches, channel counts around the blocks of
+16).  Tolerances of the scope table: forward rel. 1e-5, gradients rel. 1e-4 (fp32)."""
+import random
+
+import pytest
+import torch
+
+import oracle
+from cases import make_problem, rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def _random_shape(rng, ndim):
+    # row lengths: multiples of 4 (specialised kernels) and others (shape-generic kernels)
+    w = rng.choice([rng.randrange(32, 300), 4 * rng.randrange(16, 140), 64, 128, 256, 260, 512, 1024, 1028])
+    if ndim == 2:
+        size = (rng.randrange(1, 48), w)
+    else:
+        w = min(w, 260)
+        size = (rng.randrange(1, 12), rng.randrange(1, 14), w)
+    d = rng.randrange(1, min(min(size), 10) + 1)
+    c_in = rng.choice([1, 2, 3, 7, 15, 16, 17, 31, 32, 33, 40])
+    if ndim == 3:
+        c_in = min(c_in, 33)
+    width = rng.choice([1, 1, 1, 2])
+    batch = rng.choice([1, 1, 2, 3])
+    return (batch, c_in, width, size, d)
+
+
+def _cases(seed, n):
+    rng = random.Random(seed)
+    return [_random_shape(rng, rng.choice([2, 2, 3])) for _ in range(n)]
+
+
+@pytest.mark.parametrize("shape", _cases(2024, 40), ids=lambda s: "B%d-C%d-w%d-%s-d%d" % (
+    s[0], s[1], s[2], "x".join(map(str, s[3])), s[4]))
+def test_random_operator_problems(shape):
+    from msd_pytorch_amd import msd_custom_convolutions as cc
+    ref = make_problem(shape, torch.float32, seed=7)
+    dev = make_problem(shape, torch.float32, device="cuda", seed=7)
+    d = ref["d"]
+    # forward with ReLU, then the three ReLU backward operators (accumulating)
+    oracle.conv_relu_forward(ref["x"], ref["k"], ref["bias"], ref["y"], d)
+    cc.conv_relu_forward(dev["x"], dev["k"], dev["bias"], dev["y"], d)
+    assert rel_err(dev["stack"], ref["stack"]) <= 1e-5, "conv_relu_forward"
+    dev["y"].copy_(ref["y"])                    # same mask on both sides
+    want_gk, want_gb = torch.ones_like(ref["k"]), torch.full_like(ref["bias"], -1.0)
+    oracle.conv_relu_backward_x(ref["y"], ref["gy"], ref["k"], ref["gx"], d)
+    oracle.conv_relu_backward_k(ref["y"], ref["gy"], ref["x"], want_gk, d)
+    oracle.conv_relu_backward_bias(ref["y"], ref["gy"], want_gb)
+    got_gk, got_gb = torch.ones_like(dev["k"]), torch.full_like(dev["bias"], -1.0)
+    cc.conv_relu_backward_x(dev["y"], dev["gy"], dev["k"], dev["gx"], d)
+    cc.conv_relu_backward_k(dev["y"], dev["gy"], dev["x"], got_gk, d)
+    cc.conv_relu_backward_bias(dev["y"], dev["gy"], got_gb)
+    torch.cuda.synchronize()
+    assert rel_err(dev["gstack"], ref["gstack"]) <= 1e-4, "conv_relu_backward_x"
+    assert rel_err(got_gk, want_gk) <= 1e-4, "conv_relu_backward_k"
+    # a bias gradient is one long sum per channel, which may cancel to almost nothing: the
+    # error is then measured against a hundredth of the sum of the magnitudes at least
+    terms = (ref["gy"] * (ref["y"] > 0)).abs().double().sum(dim=[0] + list(range(2, ref["gy"].dim())))
+    floor = 0.01 * terms.max().item()
+    diff = (got_gb.double().cpu() - want_gb.double()).abs().max().item()
+    assert diff <= 1e-4 * max(want_gb.abs().max().item(), floor), "conv_relu_backward_bias"
+    # the three plain operators in one call
+    ref2 = make_problem(shape, torch.float32, seed=8)
+    dev2 = make_problem(shape, torch.float32, device="cuda", seed=8)
+    want_gk, want_gb = torch.zeros_like(ref2["k"]), torch.zeros_like(ref2["bias"])
+    oracle.conv_backward_x(ref2["gy"], ref2["k"], ref2["gx"], d)
+    oracle.conv_backward_k(ref2["gy"], ref2["x"], want_gk, d)
+    oracle.conv_backward_bias(ref2["gy"], want_gb)
+    got_gk, got_gb = torch.zeros_like(dev2["k"]), torch.zeros_like(dev2["bias"])
+    cc.conv_backward_xkb(dev2["gy"], dev2["x"], dev2["k"], dev2["gx"], got_gk, got_gb, d)
+    torch.cuda.synchronize()
+    assert rel_err(dev2["gstack"], ref2["gstack"]) <= 1e-4, "conv_backward_xkb grad_input"
+    assert rel_err(got_gk, want_gk) <= 1e-4, "conv_backward_xkb grad_kernel"
+    floor = 0.01 * ref2["gy"].abs().double().sum(dim=[0] + list(range(2, ref2["gy"].dim()))).max().item()
+    diff = (got_gb.double().cpu() - want_gb.double()).abs().max().item()
+    assert diff <= 1e-4 * max(want_gb.abs().max().item(), floor), "conv_backward_xkb grad_bias"
+
+
+def _block_cases(seed, n):
+    rng = random.Random(seed)
+    out = []
+    for _ in range(n):
+        ndim = rng.choice([2, 2, 3])
+        w = rng.choice([4 * rng.randrange(16, 100), 64, 128, 256, 132, rng.randrange(33, 200)])
+        size = (rng.randrange(4, 40), w) if ndim == 2 else (rng.randrange(3, 9), rng.randrange(3, 10), min(w, 132))
+        depth = rng.choice([1, 2, 5, 9, 17, 20])
+        width = rng.choice([1, 1, 2])
+        dil = [rng.randrange(1, min(min(size), 10) + 1) for _ in range(depth)]
+        out.append((ndim, size, rng.choice([1, 2, 3]), width, depth, rng.choice([1, 2]), dil))
+    return out
+
+
+@pytest.mark.parametrize("case", _block_cases(77, 16), ids=lambda c: "%dd-%s-c%d-w%d-depth%d-B%d" % (
+    c[0], "x".join(map(str, c[1])), c[2], c[3], c[4], c[5]))
+def test_random_blocks(case):
+    from msd_pytorch_amd.msd_block import msd_block
+    ndim, size, c_in, width, depth, batch, dil = case
+    gen = torch.Generator().manual_seed(5)
+    x = torch.randn(batch, c_in, *size, generator=gen)
+    ws = [torch.randn(width, c_in + width * i, *([3] * ndim), generator=gen) *
+          (2.0 / (3 ** ndim * (c_in + width * i))) ** 0.5 for i in range(depth)]
+    bias = torch.randn(depth * width, generator=gen) * 0.1
+    g = torch.randn(batch, c_in + depth * width, *size, generator=gen)
+    want = oracle.block_forward(x.double(), dil, bias.double(), [w.double() for w in ws])
+    xd = x.cuda().requires_grad_(True)
+    bd = bias.cuda().requires_grad_(True)
+    wd = [w.cuda().requires_grad_(True) for w in ws]
+    got = msd_block(xd, dil, bd, *wd)
+    got.backward(g.cuda())
+    torch.cuda.synchronize()
+    assert rel_err(got, want) <= 1e-5
+    # The backward oracle takes its ReLU masks from the stack the GPU computed: an activation
+    # within rounding of zero may have the other sign in double precision, and one flipped
+    # mask in an upper layer changes every gradient below it by far more than the tolerance.
+    want_gx, want_gb, want_gw = oracle.block_backward(got.detach().double().cpu(), g.double(), dil, bias.double(),
+                                                      [w.double() for w in ws])
+    assert rel_err(xd.grad, want_gx) <= 1e-4
+    assert rel_err(bd.grad, want_gb) <= 1e-4
+    assert max(rel_err(a.grad, b) for a, b in zip(wd, want_gw)) <= 1e-4
