@@ -53,7 +53,7 @@ def make_problem(shape, dtype, device="cpu", seed=0):
 
 
 def rel_err(got, want):
-    """max |got - want| / max |want| (the parity measure of the scope table)."""
+    """max |got - want| / max |want|: the parity measure of every tolerance in these tests."""
     got, want = got.detach().double().cpu(), want.detach().double().cpu()
     scale = max(want.abs().max().item(), 1e-30)
     return (got - want).abs().max().item() / scale

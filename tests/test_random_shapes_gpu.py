@@ -1,7 +1,7 @@
 """Seeded random problems against the CPU oracle: operators and whole blocks at shapes nobody
 picked by hand (ragged rows, row lengths around the kernels' limits, dilations up to the
 smallest extent, one or two output channels, batches, channel counts around the blocks of
-16).  Tolerances of the scope table: forward rel. 1e-5, gradients rel. 1e-4 (fp32)."""
+16).  Tolerances: forward rel. 1e-5, gradients rel. 1e-4 (fp32)."""
 import random
 
 import pytest
