@@ -1,6 +1,7 @@
 """Properties that do not need the oracle, checked at the image sizes of the
-headline workloads (1024 x 1024 and 128^3): adjoint identities, constants,
-linearity, and agreement of the specialised kernels with the shape-generic ones."""
+workloads (1024 x 1024 and 128^3; 4 x 512^2, 2048^2 with two output channels and
+256^3 for the last one): adjoint identities, constants, linearity, and agreement
+of the specialised kernels with the shape-generic ones."""
 import pytest
 import torch
 
@@ -92,3 +93,44 @@ def test_specialised_kernels_agree_with_generic_ones(cc, size, C, d):
     assert rel_err(g1, g0) <= 1e-4
     assert rel_err(gk1, gk0) <= 1e-4
     assert rel_err(gb1, gb0) <= 1e-4
+
+
+# the image sizes of the other workloads: 4 x 512^2 (batch), 2048^2 with two output
+# channels per layer, 256^3
+OTHER_SIZES = [(4, (512, 512), 6, 1), (1, (2048, 2048), 4, 2), (1, (256, 256, 256), 3, 1), (2, (512, 512), 18, 2)]
+
+
+@pytest.mark.parametrize("batch,size,C,width", OTHER_SIZES)
+@pytest.mark.parametrize("d", [2, 9])
+def test_other_workload_sizes_specialised_against_generic(cc, batch, size, C, width, d):
+    # every operator, and the three plain backward operators as one call, on both kernel families
+    from msd_pytorch_amd import _native
+    lib = _native.load()
+    torch.manual_seed(2)
+    nd = len(size)
+    stack = torch.randn(batch, C + width, *size, device="cuda")
+    grads = torch.randn(batch, C + width, *size, device="cuda")
+    k = torch.randn(width, C, *([3] * nd), device="cuda") * 0.2
+    bias = torch.randn(width, device="cuda") * 0.1
+    results = []
+    try:
+        for path in (1, 0):
+            lib.msd_set_kernel_path(path)
+            s, g, g2 = stack.clone(), grads.clone(), grads.clone()
+            gk, gb = torch.zeros_like(k), torch.zeros_like(bias)
+            gk2, gb2 = torch.zeros_like(k), torch.zeros_like(bias)
+            cc.conv_relu_forward(s[:, :C], k, bias, s[:, C:], d)
+            # both families mask with the activations of the first forward pass: one that is
+            # within rounding of zero may come out with the other sign from the other kernel
+            m = results[0][0] if results else s
+            cc.conv_relu_backward_x(m[:, C:], g[:, C:], k, g[:, :C], d)
+            cc.conv_relu_backward_kb(m[:, C:], g[:, C:], m[:, :C], gk, gb, d)
+            cc.conv_backward_xkb(g2[:, C:], s[:, :C], k, g2[:, :C], gk2, gb2, d)
+            results.append((s, g, gk, gb, g2, gk2, gb2))
+    finally:
+        lib.msd_set_kernel_path(0)
+    generic, fast = results
+    for name, a, b, tol in zip(("forward", "backward_x", "backward_k", "backward_bias", "xkb grad_input",
+                                "xkb grad_kernel", "xkb grad_bias"), fast, generic,
+                               (1e-5, 1e-4, 1e-4, 1e-4, 1e-4, 1e-4, 1e-4)):
+        assert rel_err(a, b) <= tol, name
