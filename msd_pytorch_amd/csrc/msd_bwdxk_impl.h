@@ -17,8 +17,8 @@
 //              tile and reads 4-voxel groups of row `tap` back per instruction;
 //   B operand  lane (channel j, voxel group k) loads x[c0 + j][16 s + 4 k ...+3] straight
 //              from memory as one 16-byte access: the layout change costs nothing.
-// The channel loop is software-pipelined in stages of 32 or 64 of the wave's voxels for
-// 16 channels of x plus 8 or 4 channels of grad_input: the loads of the next stage are
+// The channel loop is software-pipelined in stages of 16 to 64 of the wave's voxels for
+// 16 channels of x plus 2 to 8 channels of grad_input: the loads of the next stage are
 // issued before the arithmetic of the current one, into the other of two register sets.
 // Partial sums of the weight gradient stay in registers over all row tiles of a
 // workgroup, are added over its waves in LDS and leave as one column-major row per
@@ -88,7 +88,10 @@ void bwd_rows_fused(const Args a, const float *__restrict__ gyp, const float *__
     constexpr int K = Taps<NDIM>::K, NPQ = RowTaps<NDIM>::NPQ;
     constexpr int KR = WOUT * K;                  // rows of the A tile: (output channel, tap)
     constexpr int TG = (KR + 15) / 16;            // groups of 16 such rows
-    constexpr int NSS = V == 1 ? (NCB == 4 ? 1 : 2) : 4;   // 16-voxel MFMA groups per pipeline stage
+    // 16-voxel MFMA groups per pipeline stage, by measurement: 32 voxels in 2D with four voxels
+    // per lane and in 3D, 16 voxels for the 64-channel 3D instance (which then fits the
+    // registers of three workgroups per CU), 64 voxels with two voxels per lane
+    constexpr int NSS = V == 1 ? (NCB == 4 ? 1 : 2) : (V == 4 ? 2 : 4);
     constexpr int H = 4 * V / NSS;                // stages per block of 16 channels (even)
     constexpr int NCS = kChanBlock / H;           // grad_input channels per stage
     constexpr int ASTRIDE = ATile<NDIM, V, WOUT>::kStride;
