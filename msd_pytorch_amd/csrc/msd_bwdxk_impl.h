@@ -68,9 +68,9 @@ struct Args {
 };
 
 // Workgroups (of four waves) that are resident per CU: the 3D kernel with one voxel per lane
-// and at most 64 channels per chunk fits 168 registers (the 64-channel one with pipeline
-// stages of 16 voxels instead of 32), so three of them share a CU; the others need up to
-// 256 registers, which leaves room for two.
+// and at most 64 channels per chunk fits 168 registers (with pipeline stages of 16 voxels),
+// so three of them share a CU; the others need up to 256 registers, which leaves room for
+// two.  (128 registers for four per CU cost 22 to 30 spilled registers and 12 % of the speed.)
 template <int NDIM, int V, int NCB, int WOUT> constexpr int resident_per_cu()
 {
     return (NDIM == 3 && V == 1 && WOUT == 1 && NCB <= 4) ? 3 : 2;
@@ -89,9 +89,9 @@ void bwd_rows_fused(const Args a, const float *__restrict__ gyp, const float *__
     constexpr int KR = WOUT * K;                  // rows of the A tile: (output channel, tap)
     constexpr int TG = (KR + 15) / 16;            // groups of 16 such rows
     // 16-voxel MFMA groups per pipeline stage, by measurement: 32 voxels in 2D with four voxels
-    // per lane and in 3D, 16 voxels for the 64-channel 3D instance (which then fits the
-    // registers of three workgroups per CU), 64 voxels with two voxels per lane
-    constexpr int NSS = V == 1 ? (NCB == 4 ? 1 : 2) : (V == 4 ? 2 : 4);
+    // per lane, 16 voxels in 3D up to 64 channels per chunk (these instances then fit the
+    // registers of three workgroups per CU without spills), 64 voxels with two voxels per lane
+    constexpr int NSS = V == 1 ? (NCB <= 4 ? 1 : 2) : (V == 4 ? 2 : 4);
     constexpr int H = 4 * V / NSS;                // stages per block of 16 channels (even)
     constexpr int NCS = kChanBlock / H;           // grad_input channels per stage
     constexpr int ASTRIDE = ATile<NDIM, V, WOUT>::kStride;
