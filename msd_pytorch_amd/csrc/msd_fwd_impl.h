@@ -268,7 +268,7 @@ hipError_t launch(const Geom &g, const View<const float> &x, const float *k, con
                   const View<float> &out, hipStream_t s)
 {
     Lattice lt;
-    if (!make_lattice(g, V, RZ, RY, knob(kKnobFwdSplit, NDIM == 3 ? 4 : 2), &lt)) return hipErrorInvalidConfiguration;
+    if (!make_lattice(g, V, RZ, RY, knob(kKnobFwdSplit, 2), &lt)) return hipErrorInvalidConfiguration;
     const int remap = knob(kKnobXcdRemap, 1);
     const dim3 grid(remap ? xcd_grid(lt.ntiles) : lt.ntiles, g.B, 1);
     const size_t lds = (size_t)lt.ks * 3 * V * lt.lpr * sizeof(float);
