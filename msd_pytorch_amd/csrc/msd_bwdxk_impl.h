@@ -70,7 +70,8 @@ struct Args {
 // Workgroups (of four waves) that are resident per CU: the 3D kernel with one voxel per lane
 // and at most 64 channels per chunk fits 168 registers (with pipeline stages of 16 voxels),
 // so three of them share a CU; the others need up to 256 registers, which leaves room for
-// two.  (128 registers for four per CU cost 22 to 30 spilled registers and 12 % of the speed.)
+// two.  (Four per CU are slower, by 2 % at 16 channels even where the 128 registers they
+// leave cost only six spilled registers: three is where the gain ends.)
 template <int NDIM, int V, int NCB, int WOUT> constexpr int resident_per_cu()
 {
     return (NDIM == 3 && V == 1 && WOUT == 1 && NCB <= 4) ? 3 : 2;
@@ -234,7 +235,10 @@ void bwd_rows_fused(const Args a, const float *__restrict__ gyp, const float *__
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
-        mfma4 acc[TG][2];                         // two independent accumulation chains per tap group
+        // Accumulation chains per tap group: two where there is one group (dependent matrix
+        // instructions would wait for each other), one where the groups already alternate.
+        constexpr int NCH = TG >= 2 ? 1 : 2;
+        mfma4 acc[TG][NCH];
         // weight gradient of one stage: 4 * NSS * TG matrix instructions
         auto stage_k = [&](int cb, int h, float (&kk)[NSS][4]) {
             const int chl = c0 + cb * kChanBlock + mj;
@@ -252,7 +256,8 @@ void bwd_rows_fused(const Args a, const float *__restrict__ gyp, const float *__
                     const float bv = keep ? kk[j][e] : 0.f;
 #pragma unroll
                     for (int tg = 0; tg < TG; tg++)
-                        acc[tg][e & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[tg][e], bv, acc[tg][e & 1], 0, 0, 0);
+                        acc[tg][e % NCH] =
+                            __builtin_amdgcn_mfma_f32_16x16x4f32(av[tg][e], bv, acc[tg][e % NCH], 0, 0, 0);
                 }
             }
         };
@@ -328,7 +333,9 @@ void bwd_rows_fused(const Args a, const float *__restrict__ gyp, const float *__
             const int cb = block_of(st), h = st % H;
             load_stage(cb, h + 1, kb, gb);
 #pragma unroll
-            for (int tg = 0; tg < TG; tg++) acc[tg][0] = acc[tg][1] = mfma4{0.f, 0.f, 0.f, 0.f};
+            for (int tg = 0; tg < TG; tg++)
+#pragma unroll
+                for (int c = 0; c < NCH; c++) acc[tg][c] = mfma4{0.f, 0.f, 0.f, 0.f};
             stage_k(cb, h, ka);
             stage_x(cb, h, ga);
             // 2D: no test around these loads.  Loads and stores retire through one in-order
@@ -350,7 +357,9 @@ void bwd_rows_fused(const Args a, const float *__restrict__ gyp, const float *__
             for (int q = 0; q < NCB; q++)
                 if (q == cb) {
 #pragma unroll
-                    for (int tg = 0; tg < TG; tg++) D[q][tg] += acc[tg][0] + acc[tg][1];
+                    for (int tg = 0; tg < TG; tg++)
+#pragma unroll
+                        for (int c = 0; c < NCH; c++) D[q][tg] += acc[tg][c];
                 }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
