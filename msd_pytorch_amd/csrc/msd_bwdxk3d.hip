@@ -1,4 +1,4 @@
-// fused backward_x + backward_k, 3D instantiations (one file per rank so they compile in parallel).
+// fused backward_x + backward_k, 3D instantiations (one file per rank and variant so they compile in parallel).
 #include "msd_bwdxk_impl.h"
 
 namespace msd {
@@ -6,14 +6,18 @@ namespace msd {
 bool fast_backward_xkb_supported_3d(const Geom &g, const View<const float> &gy, const View<const float> &x,
                                     const View<float> &gx)
 {
-    return bwdxk::xkb_supported_nd<3>(g, gy, x, gx);
+    return bwdxk::xkb_mode<3>(g, gy, x, gx) != bwdxk::kUnsupported;
 }
 
 hipError_t fast_backward_xkb_3d(const Geom &g, const View<const float> &gy, const View<const float> &x, const float *k,
                                 const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws,
                                 hipStream_t s, ReduceJob *defer)
 {
-    return bwdxk::xkb_nd<3>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
+    switch (bwdxk::xkb_mode<3>(g, gy, x, gx)) {
+    case bwdxk::kPlain: return bwdxk::xkb_nd<3, false>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
+    case bwdxk::kLong: return fast_backward_xkb_3d_long(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
+    default: return hipErrorInvalidConfiguration;
+    }
 }
 
 }  // namespace msd

@@ -1,0 +1,13 @@
+// fused backward_x + backward_k, 3D instantiations of the variant for long rows and big stacks.
+#include "msd_bwdxk_impl.h"
+
+namespace msd {
+
+hipError_t fast_backward_xkb_3d_long(const Geom &g, const View<const float> &gy, const View<const float> &x,
+                                     const float *k, const View<float> &gx, const PostMask &pm, float *gk, float *gb,
+                                     float *ws, hipStream_t s, ReduceJob *defer)
+{
+    return bwdxk::xkb_nd<3, true>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
+}
+
+}  // namespace msd

@@ -65,6 +65,7 @@ struct Args {
     Plane gx;            // grad_input channels (written through a cast)
     int mask_from;       // activations (viewed like grad_input) mask the channels >= mask_from
     int want_bias;
+    RowSegments sg;      // LONG instances, 2D
 };
 
 // Workgroups (of four waves) that are resident per CU: the 3D kernel with one voxel per lane
@@ -77,7 +78,12 @@ template <int NDIM, int V, int NCB, int WOUT> constexpr int resident_per_cu()
     return (NDIM == 3 && V == 1 && WOUT == 1 && NCB <= 4) ? 3 : 2;
 }
 
-template <int NDIM, int V, int NCB, int WOUT>
+// LONG: the variant for what the plain kernel's 32-bit lane offsets and whole-row teams do
+// not reach.  The first channel of each block of 16 moves into the uniform base of the x
+// loads (so the stack may be of any size), and 2D rows longer than a workgroup covers are cut
+// into segments, staged with a halo of `dil` values on either side.  It is a separate
+// instance because even its few extra scalar instructions per stage cost the plain one 1-4 %.
+template <int NDIM, int V, int NCB, int WOUT, bool LONG>
 __global__ __launch_bounds__(kThreads, (resident_per_cu<NDIM, V, NCB, WOUT>()))
 void bwd_rows_fused(const Args a, const float *__restrict__ gyp, const float *__restrict__ xp,
                     float *__restrict__ gxp, const float *__restrict__ actp, const float *__restrict__ kw,
@@ -103,8 +109,12 @@ void bwd_rows_fused(const Args a, const float *__restrict__ gyp, const float *__
     const int wave = __builtin_amdgcn_readfirstlane(tid / kWave), wl = tid % kWave;
     const int mk = wl / 16, mj = wl % 16;         // MFMA k (voxel group) and i/j (tap or channel) of this lane
     const int team = tid / rt.lpr, lane = tid % rt.lpr;
-    float *S = lds + (size_t)team * WOUT * NPQ * V * rt.lpr;
-    float *AT = lds + (size_t)rt.rpw * WOUT * NPQ * V * rt.lpr + (size_t)wave * ATile<NDIM, V, WOUT>::kFloats;
+    // segments (rt.segs > 1): a tile is one segment of one row
+    constexpr bool SEG = LONG && NDIM == 2;
+    const bool segmented = SEG && a.sg.segs > 1;  // uniform
+    const int rs = V * rt.lpr + (SEG ? a.sg.halo : 0);   // floats per staged row
+    float *S = lds + (size_t)team * WOUT * NPQ * rs;
+    float *AT = lds + (size_t)rt.rpw * WOUT * NPQ * rs + (size_t)wave * ATile<NDIM, V, WOUT>::kFloats;
     for (int i = wl; i < ASTRIDE; i += kWave) AT[KR * ASTRIDE + i] = 0.f;
 
     const int c0 = blockIdx.z * NCB * kChanBlock;
@@ -127,9 +137,9 @@ void bwd_rows_fused(const Args a, const float *__restrict__ gyp, const float *__
         for (int tg = 0; tg < TG; tg++) D[cb][tg] = mfma4{0.f, 0.f, 0.f, 0.f};
 
     const int lb = block_for_xcd(blockIdx.x, gridDim.x, a.remap);
-    const int x0 = lane * V;
-    const int xc = min(x0, g.W - V);
-    const int kx = (lane - wl) * V + 4 * mk;      // first voxel of this lane's MFMA groups, + 16 s
+    const int x0_row = lane * V;
+    const int xc_row = min(x0_row, g.W - V);
+    const int kx_row = (lane - wl) * V + 4 * mk;  // first voxel of this lane's MFMA groups, + 16 s
     int arow[TG];                                 // this lane's row of the A tile (the zero row past K taps)
 #pragma unroll
     for (int tg = 0; tg < TG; tg++) arow[tg] = min(tg * 16 + mj, KR) * ASTRIDE + 4 * mk;
@@ -137,7 +147,12 @@ void bwd_rows_fused(const Args a, const float *__restrict__ gyp, const float *__
     // Position of the lane's row, advanced from tile to tile without divisions: the row groups
     // of a workgroup are consecutive.
     int grp = a.group_step == 1 ? lb * a.tiles_per_wg : lb;
-    int gi = grp % a.ngroups, b = grp / a.ngroups;            // uniform: group within the image, batch index
+    int seg = 0, rg = grp;                                    // uniform: segment of the row, row group
+    if constexpr (SEG) {
+        seg = grp % a.sg.segs;
+        rg = grp / a.sg.segs;
+    }
+    int gi = rg % a.ngroups, b = rg / a.ngroups;              // uniform: group within the image, batch index
     int row = gi * rt.rpw + team;
     int y = row % g.H, z = row / g.H;
 
@@ -145,12 +160,17 @@ void bwd_rows_fused(const Args a, const float *__restrict__ gyp, const float *__
         if (grp >= a.total_groups) break;         // uniform over the workgroup
         int xsc = a.x.sc, gsc = a.gx.sc;
         asm volatile("" : "+s"(xsc), "+s"(gsc));  // keeps per-channel addresses from being hoisted out of the loop
+        const int xs = SEG ? seg * V * rt.lpr : 0;    // first voxel of the segment
+        const int x0 = SEG ? xs + x0_row : x0_row;
+        const int xc = SEG ? x0 : xc_row;             // (whole segments only: never past the row)
+        const int kx = SEG ? xs + kx_row : kx_row;
         const bool rowok = row < rt.nrows;        // teams past the last row work on it again and store nothing
         const bool act = rowok && x0 < g.W;
         const int zc = rowok ? z : g.D - 1, yc = rowok ? y : g.H - 1;
         // Addresses are a wave-uniform 64-bit base (scalar registers) plus a 32-bit byte offset
         // per lane, the form the memory instructions take directly.  x: the lane's channel is
-        // part of the offset; grad_input and activations: the channel is part of the base.
+        // part of the offset (LONG: its channel within the block of 16 only); grad_input and
+        // activations: the channel is part of the base.
         const uint64_t xbase = reinterpret_cast<uint64_t>(xp + (int64_t)b * a.x.sb);
         const uint32_t xrow = (uint32_t)(zc * a.x.sz + yc * a.x.sy);
         const uint64_t gbase = reinterpret_cast<uint64_t>(gxp + (int64_t)b * a.gx.sb);
@@ -172,10 +192,19 @@ void bwd_rows_fused(const Args a, const float *__restrict__ gyp, const float *__
             // (redefining the lane offset keeps its widening to 64 bits next to the loads, where
             // it is free; hoisted out of the loop it would make every address a vector addition)
             asm volatile("" : "+v"(goff));
-            const uint32_t xch = (uint32_t)min(c0 + cb * kChanBlock + mj, g.C - 1) * (uint32_t)xsc + xrow;
+            if constexpr (LONG) {
+                const int cb0 = c0 + cb * kChanBlock;
+                const uint64_t xb = xbase + (uint64_t)(uint32_t)cb0 * (uint32_t)(4 * xsc);
+                const uint32_t xch = (uint32_t)min(mj, g.C - 1 - cb0) * (uint32_t)xsc + xrow;
 #pragma unroll
-            for (int j = 0; j < NSS; j++)
-                load_global_vec<4>(xbase, 4u * (xch + (uint32_t)min(kx + 16 * (h * NSS + j), g.W - 4)), kk[j]);
+                for (int j = 0; j < NSS; j++)
+                    load_global_vec<4>(xb, 4u * (xch + (uint32_t)min(kx + 16 * (h * NSS + j), g.W - 4)), kk[j]);
+            } else {
+                const uint32_t xch = (uint32_t)min(c0 + cb * kChanBlock + mj, g.C - 1) * (uint32_t)xsc + xrow;
+#pragma unroll
+                for (int j = 0; j < NSS; j++)
+                    load_global_vec<4>(xbase, 4u * (xch + (uint32_t)min(kx + 16 * (h * NSS + j), g.W - 4)), kk[j]);
+            }
 #pragma unroll
             for (int j = 0; j < NCS; j++) {
                 const int ci = max(min(c0 + cb * kChanBlock + h * NCS + j, cx_end - 1), 0);
@@ -192,15 +221,21 @@ void bwd_rows_fused(const Args a, const float *__restrict__ gyp, const float *__
             const View<const float> none{nullptr, 0, 0, 0, 0, 0};
             const View<const float> gyv{gyp, a.gy.sb, a.gy.sc, a.gy.sz, a.gy.sy, 1};
             float own[WOUT][NPQ][V];
-            stage_source_rows<NDIM, false, WOUT, V>(g, rt, none, gyv, b, zc, yc, lane, act, S, own);
+            if (segmented) {
+                if constexpr (SEG) stage_source_segment<WOUT, V>(g, rt, a.sg, gyv, b, yc, xs, lane, rowok, S, own);
+            } else {
+                stage_source_rows<NDIM, false, WOUT, V>(g, rt, none, gyv, b, zc, yc, lane, act, S, own);
+            }
             // per voxel: all LDS reads first, so that their latencies overlap, then the sums
 #pragma unroll
             for (int i = 0; i < V; i++) {
-                const SideTaps<V> side(min(x0 + i, g.W - 1), g.W, g.dil, rt.lpr);
+                const SideTaps<V> side = segmented
+                                             ? SideTaps<V>(x0 + i, g.W, g.dil, rt.lpr, xs, V * rt.lpr)
+                                             : SideTaps<V>(min(x0 + i, g.W - 1), g.W, g.dil, rt.lpr);
                 float ra[WOUT * NPQ][4];
 #pragma unroll
                 for (int pq = 0; pq < WOUT * NPQ; pq++) {
-                    const float *srow = S + (size_t)pq * V * rt.lpr;
+                    const float *srow = S + (size_t)pq * rs;
                     ra[pq][0] = srow[side.i0a];
                     ra[pq][1] = srow[side.i0b];
                     ra[pq][2] = srow[side.i2a];
@@ -366,10 +401,15 @@ void bwd_rows_fused(const Args a, const float *__restrict__ gyp, const float *__
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         // next row group
-        if (a.group_step != 1) {                  // uniform
+        if (a.group_step != 1 || SEG) {           // uniform
             grp += a.group_step;
-            gi = grp % a.ngroups;
-            b = grp / a.ngroups;
+            rg = grp;
+            if constexpr (SEG) {
+                seg = grp % a.sg.segs;
+                rg = grp / a.sg.segs;
+            }
+            gi = rg % a.ngroups;
+            b = rg / a.ngroups;
             row = gi * rt.rpw + team;
             y = row % g.H;
             z = row / g.H;
@@ -436,10 +476,10 @@ void bwd_rows_fused(const Args a, const float *__restrict__ gyp, const float *__
 }
 
 template <int NDIM, int V, int NCB, int WOUT>
-size_t lds_bytes(const RowTeams &rt)
+size_t lds_bytes(const RowTeams &rt, const RowSegments &sg)
 {
     constexpr int TG = (WOUT * Taps<NDIM>::K + 15) / 16;
-    const size_t main_loop = ((size_t)rt.rpw * WOUT * RowTaps<NDIM>::NPQ * V * rt.lpr +
+    const size_t main_loop = ((size_t)rt.rpw * WOUT * RowTaps<NDIM>::NPQ * (V * rt.lpr + sg.halo) +
                               (size_t)kWaves * ATile<NDIM, V, WOUT>::kFloats) * 4;
     const size_t epilogue = (size_t)kWaves * NCB * TG * 4 * kWave * 4;
     return std::max(main_loop, epilogue);
@@ -457,26 +497,28 @@ inline bool small_strides(const Geom &g, const View<T> &v)
 // Usable with V voxels per lane: whole waves per row, rows fit a 256-lane workgroup,
 // 16-byte accesses to x and V-wide ones to the other tensors aligned.
 template <int NDIM>
-bool fits(const Geom &g, int V, const View<const float> &gy, const View<const float> &x, const View<float> &gx)
+bool fits(const Geom &g, int V, const View<const float> &gy, const View<const float> &x, const View<float> &gx,
+          bool lng)
 {
     RowTeams rt;
-    if (g.W % 4 != 0 || !make_row_teams(g, V, &rt)) return false;
+    RowSegments sg;
+    if (g.W % 4 != 0 || !make_row_teams(g, V, &rt, lng && NDIM == 2 ? &sg : nullptr)) return false;
     if (rt.lpr % kWave != 0 || rt.lpr * rt.rpw > kThreads) return false;
     return rows_aligned(x, g.W, 4) && rows_aligned(gy, g.W, V) && rows_aligned(gx, g.W, V);
 }
 
 template <int NDIM>
 int choose_vec(const Geom &g, int vmax, const View<const float> &gy, const View<const float> &x,
-               const View<float> &gx)
+               const View<float> &gx, bool lng)
 {
     for (int v = NDIM == 3 ? 2 : 4; v >= 1; v /= 2) {
         if (v > vmax) continue;
-        if (fits<NDIM>(g, v, gy, x, gx)) return v;
+        if (fits<NDIM>(g, v, gy, x, gx, lng)) return v;
     }
     return 0;
 }
 
-template <int NDIM, int V, int NCB, int WOUT>
+template <int NDIM, int V, int NCB, int WOUT, bool LONG>
 hipError_t launch(const Geom &g, const View<const float> &gy, const View<const float> &x, const float *k,
                   const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws, hipStream_t s,
                   ReduceJob *defer)
@@ -484,11 +526,12 @@ hipError_t launch(const Geom &g, const View<const float> &gy, const View<const f
     constexpr int K = Taps<NDIM>::K;
     Args a;
     a.g = g;
-    make_row_teams(g, V, &a.rt);
+    a.sg = RowSegments{1, 0};
+    make_row_teams(g, V, &a.rt, LONG && NDIM == 2 ? &a.sg : nullptr);
     // a deferred reduction brings its own region for the partial sums (defer->part)
     float *part = defer ? const_cast<float *>(defer->part) : ws + backward_k_mask_floats(g);
     a.ngroups = (a.rt.nrows + a.rt.rpw - 1) / a.rt.rpw;
-    const int64_t total = (int64_t)a.ngroups * g.B;
+    const int64_t total = (int64_t)a.ngroups * a.sg.segs * g.B;
     a.remap = knob(kKnobXcdRemap, 1);
     // as many workgroups as are resident at once (256 CUs): the grid then runs as one round
     const int64_t max_wgs = std::min<int64_t>(
@@ -512,8 +555,8 @@ hipError_t launch(const Geom &g, const View<const float> &gy, const View<const f
     a.mask_from = pm.from;
     a.want_bias = gb != nullptr;
     const int chunks = (g.C + NCB * kChanBlock - 1) / (NCB * kChanBlock);
-    const size_t lds = lds_bytes<NDIM, V, NCB, WOUT>(a.rt);
-    hipLaunchKernelGGL((bwd_rows_fused<NDIM, V, NCB, WOUT>), dim3(rows, 1, chunks), dim3(a.rt.lpr * a.rt.rpw), lds, s, a,
+    const size_t lds = lds_bytes<NDIM, V, NCB, WOUT>(a.rt, a.sg);
+    hipLaunchKernelGGL((bwd_rows_fused<NDIM, V, NCB, WOUT, LONG>), dim3(rows, 1, chunks), dim3(a.rt.lpr * a.rt.rpw), lds, s, a,
                        gy.p, x.p, gx.p, actp, k, part);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
@@ -527,62 +570,69 @@ hipError_t launch(const Geom &g, const View<const float> &gy, const View<const f
     return hipGetLastError();
 }
 
-template <int NDIM, int V, int WOUT>
+template <int NDIM, int V, int WOUT, bool LONG>
 hipError_t pick_ncb(const Geom &g, const View<const float> &gy, const View<const float> &x, const float *k,
                     const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws, hipStream_t s,
                     ReduceJob *defer)
 {
     const int need = (g.C + kChanBlock - 1) / kChanBlock;
-    if (need <= 1) return launch<NDIM, V, 1, WOUT>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
-    if (need <= 2) return launch<NDIM, V, 2, WOUT>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
-    if (need <= 4) return launch<NDIM, V, 4, WOUT>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
-    return launch<NDIM, V, 8, WOUT>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
+    if (need <= 1) return launch<NDIM, V, 1, WOUT, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
+    if (need <= 2) return launch<NDIM, V, 2, WOUT, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
+    if (need <= 4) return launch<NDIM, V, 4, WOUT, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
+    return launch<NDIM, V, 8, WOUT, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
 }
 
 // Widest vector for two output channels (2D only): twice the gathered values per voxel must
 // still fit the registers beside the pipeline buffers.
 constexpr int kMaxVecTwoOutputs = 2;
 
-// One output channel (2D: one or two), unit x-strides, 32-bit strides, and a vector width
-// that fits.
-template <int NDIM>
-bool xkb_supported_nd(const Geom &g, const View<const float> &gy, const View<const float> &x, const View<float> &gx)
+// Lane offsets into x fit 32 bits: they span the whole stack in the plain kernel, one block
+// of 16 channels in the LONG one.
+inline bool x_offsets_fit(const Geom &g, const View<const float> &x, bool lng)
 {
-    if (g.Wd != 1 && !(NDIM == 2 && g.Wd == 2)) return false;
-    if (x.sx != 1 || gy.sx != 1 || gx.sx != 1) return false;
-    if (g.Wd == 2) {
-        if (!small_strides(g, gy) || !small_strides(g, x) || !small_strides(g, gx)) return false;
-        if ((int64_t)g.C * x.sc + (int64_t)g.D * x.sz + (int64_t)g.H * x.sy + g.W >= ((int64_t)1 << 30)) return false;
-        return choose_vec<NDIM>(g, kMaxVecTwoOutputs, gy, x, gx) != 0;
-    }
-    if (!small_strides(g, gy) || !small_strides(g, x) || !small_strides(g, gx)) return false;
-    if ((int64_t)g.C * x.sc + (int64_t)g.D * x.sz + (int64_t)g.H * x.sy + g.W >= ((int64_t)1 << 30)) return false;
-    return choose_vec<NDIM>(g, 4, gy, x, gx) != 0;
+    const int64_t channels = lng ? kChanBlock : g.C;
+    return channels * x.sc + (int64_t)g.D * x.sz + (int64_t)g.H * x.sy + g.W < ((int64_t)1 << 30);
+}
+
+enum Mode { kUnsupported = 0, kPlain = 1, kLong = 2 };
+
+// One output channel (2D: one or two), unit x-strides, 32-bit strides, and a vector width
+// that fits: with the plain kernel where it reaches, else with the LONG one.
+template <int NDIM>
+Mode xkb_mode(const Geom &g, const View<const float> &gy, const View<const float> &x, const View<float> &gx)
+{
+    if (g.Wd != 1 && !(NDIM == 2 && g.Wd == 2)) return kUnsupported;
+    if (x.sx != 1 || gy.sx != 1 || gx.sx != 1) return kUnsupported;
+    if (!small_strides(g, gy) || !small_strides(g, x) || !small_strides(g, gx)) return kUnsupported;
+    const int vmax = g.Wd == 2 ? kMaxVecTwoOutputs : 4;
+    if (x_offsets_fit(g, x, false) && choose_vec<NDIM>(g, vmax, gy, x, gx, false) != 0) return kPlain;
+    if (x_offsets_fit(g, x, true) && choose_vec<NDIM>(g, vmax, gy, x, gx, true) != 0) return kLong;
+    return kUnsupported;
 }
 
 // pm.act, where pm.from < C, must be laid out like gx (same strides and 16-byte phase).
-template <int NDIM>
+template <int NDIM, bool LONG>
 hipError_t xkb_nd(const Geom &g, const View<const float> &gy, const View<const float> &x, const float *k,
                   const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws, hipStream_t s,
                   ReduceJob *defer)
 {
     // 3D: one voxel per lane keeps the 27 gathered values per voxel and the pipeline buffers in registers
     const int vmax = knob(NDIM == 3 ? kKnobBwdkVec3d : kKnobBwdkVec2d, NDIM == 3 ? 1 : 4);
-    int v = choose_vec<NDIM>(g, vmax, gy, x, gx);
-    if (v == 0) v = choose_vec<NDIM>(g, 4, gy, x, gx);
+    int v = choose_vec<NDIM>(g, vmax, gy, x, gx, LONG);
+    if (v == 0) v = choose_vec<NDIM>(g, 4, gy, x, gx, LONG);
     if constexpr (NDIM == 2) {
         if (g.Wd == 2) {
-            v = choose_vec<2>(g, std::min(vmax, kMaxVecTwoOutputs), gy, x, gx);
-            if (v == 0) v = choose_vec<2>(g, kMaxVecTwoOutputs, gy, x, gx);
-            if (v == 2) return pick_ncb<2, 2, 2>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
-            if (v == 1) return pick_ncb<2, 1, 2>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
+            v = choose_vec<2>(g, std::min(vmax, kMaxVecTwoOutputs), gy, x, gx, LONG);
+            if (v == 0) v = choose_vec<2>(g, kMaxVecTwoOutputs, gy, x, gx, LONG);
+            if (v == 2) return pick_ncb<2, 2, 2, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
+            if (v == 1) return pick_ncb<2, 1, 2, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
             return hipErrorInvalidConfiguration;
         }
-        if (v == 4) return pick_ncb<2, 4, 1>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
+        if (v == 4) return pick_ncb<2, 4, 1, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
     }
     if (g.Wd != 1) return hipErrorInvalidConfiguration;
-    if (v == 2) return pick_ncb<NDIM, 2, 1>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
-    if (v == 1) return pick_ncb<NDIM, 1, 1>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
+    if (v == 2) return pick_ncb<NDIM, 2, 1, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
+    if (v == 1) return pick_ncb<NDIM, 1, 1, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
     return hipErrorInvalidConfiguration;
 }
 

@@ -158,6 +158,14 @@ hipError_t fast_backward_xkb_2d(const Geom &g, const View<const float> &gy, cons
 hipError_t fast_backward_xkb_3d(const Geom &g, const View<const float> &gy, const View<const float> &x, const float *k,
                                 const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws,
                                 hipStream_t s, ReduceJob *defer);
+// the instances for rows longer than a workgroup covers (2D) and for stacks whose offsets do
+// not fit 32 bits; chosen by fast_backward_xkb_2d / _3d, not called directly
+hipError_t fast_backward_xkb_2d_long(const Geom &g, const View<const float> &gy, const View<const float> &x,
+                                     const float *k, const View<float> &gx, const PostMask &pm, float *gk, float *gb,
+                                     float *ws, hipStream_t s, ReduceJob *defer);
+hipError_t fast_backward_xkb_3d_long(const Geom &g, const View<const float> &gy, const View<const float> &x,
+                                     const float *k, const View<float> &gx, const PostMask &pm, float *gk, float *gb,
+                                     float *ws, hipStream_t s, ReduceJob *defer);
 
 inline bool fast_backward_xkb_supported(const Geom &g, const View<const float> &gy, const View<const float> &x,
                                         const View<float> &gx)

@@ -27,12 +27,22 @@ namespace msd {
 
 struct RowTeams {
     int V;       // voxels per lane
-    int lpr;     // lanes per row
+    int lpr;     // lanes per row (per segment of a row that is cut into segments)
     int rpw;     // rows (teams) per workgroup
     int nrows;   // D * H
 };
 
-inline bool make_row_teams(const Geom &g, int V, RowTeams *rt)
+struct RowSegments {
+    int segs;    // segments a row is cut into (1: a team owns a whole row)
+    int halo;    // floats appended to each staged row for the neighbours of a segment (0 when segs == 1)
+};
+
+constexpr int kSegmentLanes = 256;   // lanes of a team that owns a segment of a long row
+
+// With `sg`: rows longer than kSegmentLanes * V voxels are cut into segments of that length,
+// one team (and workgroup) each; the kernels that ask for it stage a halo of `dil` values on
+// either side (stage_source_segment).  2D only, whole segments only, dil <= 128.
+inline bool make_row_teams(const Geom &g, int V, RowTeams *rt, RowSegments *sg = nullptr)
 {
     const int need = (g.W + V - 1) / V;
     int lpr;
@@ -42,11 +52,21 @@ inline bool make_row_teams(const Geom &g, int V, RowTeams *rt)
     } else {
         lpr = (need + kWave - 1) / kWave * kWave;
     }
-    if (lpr > 1024) return false;
     rt->V = V;
+    rt->nrows = g.D * g.H;
+    if (sg) *sg = RowSegments{1, 0};
+    if (sg && lpr > kSegmentLanes) {
+        const int segw = kSegmentLanes * V;
+        if (g.ndim != 2 || g.W % segw != 0 || 2 * g.dil > kSegmentLanes) return false;
+        rt->lpr = kSegmentLanes;
+        rt->rpw = 1;
+        sg->segs = g.W / segw;
+        sg->halo = (2 * g.dil + 3) & ~3;         // keeps what follows the staged rows 16-byte aligned
+        return true;
+    }
+    if (lpr > 1024) return false;
     rt->lpr = lpr;
     rt->rpw = lpr >= 256 ? 1 : 256 / lpr;
-    rt->nrows = g.D * g.H;
     return true;
 }
 
@@ -197,6 +217,57 @@ __device__ __forceinline__ void stage_source_rows(const Geom &g, const RowTeams 
     __syncthreads();
 }
 
+// Segment variant of stage_source_rows (2D, no ReLU mask): the team owns voxels
+// [xs, xs + V * lpr) of row y.  A staged row holds the segment in the usual layout, then
+// `dil` values to the left of it and `dil` values to the right (zeros outside the row), which
+// the lanes 0 .. 2 dil - 1 load one each.  Ends with a workgroup barrier.
+template <int WOUT, int V>
+__device__ __forceinline__ void stage_source_segment(const Geom &g, const RowTeams &rt, const RowSegments &sg,
+                                                     const View<const float> &gy, int b, int y, int xs, int lane, bool rowok,
+                                                     float *__restrict__ S, float (&own)[WOUT][3][V])
+{
+    const AxisSources sy = adjoint_sources(y, g.H, g.dil);
+    const int rs = V * rt.lpr + sg.halo;         // floats per staged row
+    const int x0 = xs + lane * V;
+    const int h = lane;                          // halo element of this lane, if any
+    const int hx = h < g.dil ? xs - g.dil + h : xs + V * rt.lpr + (h - g.dil);
+    const bool hin = h < 2 * g.dil && hx >= 0 && hx < g.W;
+    const int hxc = min(max(hx, 0), g.W - 1);
+    const bool folds = y < g.dil || y + g.dil >= g.H;
+#pragma unroll
+    for (int co = 0; co < WOUT; co++) {
+        const float *gc = gy.p + (int64_t)b * gy.sb + (int64_t)co * gy.sc;
+        float s[3][V], sh[3];
+        auto add_row = [&](int q, int cy, bool ok, bool first) {
+            cy = min(max(cy, 0), g.H - 1);
+            const float *rowp = gc + (int64_t)cy * gy.sy;
+            float m[V];
+            load_vec<V>(rowp + x0, m);
+            const float mh = rowp[hxc];
+#pragma unroll
+            for (int i = 0; i < V; i++) s[q][i] = (first ? 0.f : s[q][i]) + (ok && rowok ? m[i] : 0.f);
+            sh[q] = (first ? 0.f : sh[q]) + (ok && rowok && hin ? mh : 0.f);
+        };
+#pragma unroll
+        for (int q = 0; q < 3; q++) add_row(q, sy.c[q][0], sy.ok[q][0], true);
+        if (folds) {
+#pragma unroll
+            for (int q = 0; q < 3; q++) add_row(q, sy.c[q][1], sy.ok[q][1], false);
+        }
+#pragma unroll
+        for (int q = 0; q < 3; q++) {
+            float *row = S + (size_t)(co * 3 + q) * rs;
+#pragma unroll
+            for (int i = 0; i < V; i++) {
+                own[co][q][i] = s[q][i];
+                row[i * rt.lpr + lane] = s[q][i];
+            }
+            if (h < 2 * g.dil) row[V * rt.lpr + h] = sh[q];
+        }
+    }
+    __syncthreads();
+}
+
 // Position of element x in a staged row.
 template <int V>
 __device__ __forceinline__ int staged_index(int x, int lpr)
@@ -225,6 +296,34 @@ struct SideTaps {
         m0b = x < dil;
         m2a = lo >= 0;
         m2b = hi >= W;
+    }
+
+    // Segment variant: x is a position in the row, the staged row holds [xs, xs + segw) in the
+    // usual layout followed by dil values to the left and dil values to the right of it.
+    __device__ __forceinline__ SideTaps(int x, int W, int dil, int lpr, int xs, int segw)
+    {
+        const int hi = x + dil, lo = x - dil;
+        auto at = [&](int p) {                   // p: position in the row that this segment stages
+            const int j = p - xs;
+            return j < 0 ? V * lpr + (j + dil) : (j >= segw ? V * lpr + dil + (j - segw) : staged_index<V>(j, lpr));
+        };
+        i0a = at(min(hi, W - 1));
+        i0b = at(min(max(dil - x - 1, 0), W - 1));
+        i2a = at(max(lo, 0));
+        i2b = at(min(max(2 * W - x - 1 - dil, 0), W - 1));
+        m0a = hi < W;
+        m0b = x < dil;
+        m2a = lo >= 0;
+        m2b = hi >= W;
+        // the mirrored sources lie in the first and the last segment only: clamp what the
+        // other segments compute for them (masked off) into the staged range
+        const int last = V * lpr + 2 * dil - 1;
+        i0b = m0b ? i0b : 0;
+        i2b = m2b ? i2b : 0;
+        i0a = min(max(i0a, 0), last);
+        i2a = min(max(i2a, 0), last);
+        i0b = min(max(i0b, 0), last);
+        i2b = min(max(i2b, 0), last);
     }
 
     __device__ __forceinline__ void read(const float *__restrict__ row, float &t0, float &t2) const

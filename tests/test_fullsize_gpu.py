@@ -103,6 +103,20 @@ OTHER_SIZES = [(4, (512, 512), 6, 1), (1, (2048, 2048), 4, 2), (1, (256, 256, 25
 @pytest.mark.parametrize("batch,size,C,width", OTHER_SIZES)
 @pytest.mark.parametrize("d", [2, 9])
 def test_other_workload_sizes_specialised_against_generic(cc, batch, size, C, width, d):
+    _compare_kernel_families(cc, batch, size, C, width, d)
+
+
+# stacks of more than 2^30 values (4 GiB): the one-pass backward kernel then addresses the input
+# channels block by block; 2048-wide rows are also cut into segments
+BIG_STACKS = [(1, (2048, 2048), 258, 2, 7), (1, (128, 128, 128), 520, 1, 3)]
+
+
+@pytest.mark.parametrize("batch,size,C,width,d", BIG_STACKS)
+def test_big_stacks_specialised_against_generic(cc, batch, size, C, width, d):
+    _compare_kernel_families(cc, batch, size, C, width, d)
+
+
+def _compare_kernel_families(cc, batch, size, C, width, d):
     # every operator, and the three plain backward operators as one call, on both kernel families
     from msd_pytorch_amd import _native
     lib = _native.load()

@@ -70,6 +70,8 @@ FUSED_BLOCK_CASES = [
     (3, (33, 31, 68), 2, 3, 2, None),      # the same in 3D, last groups ragged
     (2, (21, 128), 2, 11, 1, None, 2),     # width 2: two output channels per layer in the fused pass
     (2, (300, 132), 2, 4, 2, None, 2),     # width 2, several tiles per workgroup
+    (2, (23, 2048), 1, 5, 2, [1, 2, 9, 23, 4]),      # rows of 2 segments of 1024 voxels
+    (2, (19, 1536), 2, 3, 1, [3, 1, 10], 2),       # width 2, rows of 3 segments of 512 voxels
 ]
 
 

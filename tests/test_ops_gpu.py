@@ -174,6 +174,13 @@ SHAPES_XKB = [
     (2, 5, 2, (7, 128), 2),           # two output channels: 2 voxels per lane, 2 rows per workgroup
     (1, 35, 2, (12, 512), 5),         # two output channels, 3 channel blocks, one row per workgroup
     (1, 16, 2, (9, 68), 3),           # two output channels, one voxel per lane, exactly one channel block
+    # rows longer than one workgroup covers: cut into segments with a halo of `dilation` values
+    (1, 3, 1, (5, 2048), 1),          # 2 segments of 1024
+    (2, 18, 1, (7, 2048), 5),         # 2 channel blocks, folds in y
+    (1, 4, 1, (130, 1536), 128),      # 3 segments of 512, the largest dilation the halo takes
+    (1, 2, 1, (140, 2048), 129),      # dilation past that: the separate kernels
+    (1, 5, 2, (8, 1024), 7),          # two output channels: 2 segments of 512
+    (1, 3, 2, (4, 2048), 3),          # two output channels: 4 segments
 ]
 
 
