@@ -35,7 +35,20 @@ def _cases(seed, n):
     return [_random_shape(rng, rng.choice([2, 2, 3])) for _ in range(n)]
 
 
-@pytest.mark.parametrize("shape", _cases(2024, 40), ids=lambda s: "B%d-C%d-w%d-%s-d%d" % (
+def _wide_cases(seed, n):
+    # 2D rows longer than one workgroup covers: whole segments of 256 * V voxels (V = 4, 2 or,
+    # with two output channels, 2) and others; dilations on both sides of the halo's limit of 128
+    rng = random.Random(seed)
+    out = []
+    for _ in range(n):
+        w = rng.choice([1536, 2048, 2048, 2560, 3072, 4096, 2052])
+        h = rng.randrange(1, 160)
+        d = rng.choice([rng.randrange(1, min(h, 12) + 1), rng.randrange(1, h + 1)])
+        out.append((rng.choice([1, 2]), rng.choice([1, 3, 17]), rng.choice([1, 2]), (h, w), d))
+    return out
+
+
+@pytest.mark.parametrize("shape", _cases(2024, 40) + _wide_cases(77, 10), ids=lambda s: "B%d-C%d-w%d-%s-d%d" % (
     s[0], s[1], s[2], "x".join(map(str, s[3])), s[4]))
 def test_random_operator_problems(shape):
     from msd_pytorch_amd import msd_custom_convolutions as cc
