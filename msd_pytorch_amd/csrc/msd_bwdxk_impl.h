@@ -162,7 +162,7 @@ void bwd_rows_fused(const Args a, const float *__restrict__ gyp, const float *__
         asm volatile("" : "+s"(xsc), "+s"(gsc));  // keeps per-channel addresses from being hoisted out of the loop
         const int xs = SEG ? seg * V * rt.lpr : 0;    // first voxel of the segment
         const int x0 = SEG ? xs + x0_row : x0_row;
-        const int xc = SEG ? x0 : xc_row;             // (whole segments only: never past the row)
+        const int xc = SEG ? min(x0, g.W - V) : xc_row;
         const int kx = SEG ? xs + kx_row : kx_row;
         const bool rowok = row < rt.nrows;        // teams past the last row work on it again and store nothing
         const bool act = rowok && x0 < g.W;
@@ -198,7 +198,8 @@ void bwd_rows_fused(const Args a, const float *__restrict__ gyp, const float *__
                 const uint32_t xch = (uint32_t)min(mj, g.C - 1 - cb0) * (uint32_t)xsc + xrow;
 #pragma unroll
                 for (int j = 0; j < NSS; j++)
-                    load_global_vec<4>(xb, 4u * (xch + (uint32_t)min(kx + 16 * (h * NSS + j), g.W - 4)), kk[j]);
+                    load_global_vec4_unaligned(xb, 4u * (xch + (uint32_t)min(kx + 16 * (h * NSS + j), g.W - 4)),
+                                               kk[j]);
             } else {
                 const uint32_t xch = (uint32_t)min(c0 + cb * kChanBlock + mj, g.C - 1) * (uint32_t)xsc + xrow;
 #pragma unroll
@@ -283,6 +284,19 @@ void bwd_rows_fused(const Args a, const float *__restrict__ gyp, const float *__
                 const int s = h * NSS + j;
                 const bool vok = rowok && kx + 16 * s < g.W;
                 const bool keep = vok && chok;
+                if constexpr (LONG) {
+                    // rows need not be whole groups of four voxels here: the last group of a row
+                    // was loaded from W - 4 (inside the row), `shift` voxels early; move its
+                    // values down and fill with zeros
+                    // (selects, no branch: nothing in the channel loop depends on the lane)
+                    const int shift = kx + 16 * s - (g.W - 4);
+                    const float r[8] = {kk[j][0], kk[j][1], kk[j][2], kk[j][3], 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        kk[j][e] = shift <= 0 ? r[e]
+                                              : (shift == 1 ? r[e + 1]
+                                                            : (shift == 2 ? r[e + 2] : (shift == 3 ? r[e + 3] : 0.f)));
+                }
                 f32x4 av[TG];
 #pragma unroll
                 for (int tg = 0; tg < TG; tg++) av[tg] = *reinterpret_cast<const f32x4 *>(AT + arow[tg] + 16 * s);
@@ -502,9 +516,11 @@ bool fits(const Geom &g, int V, const View<const float> &gy, const View<const fl
 {
     RowTeams rt;
     RowSegments sg;
-    if (g.W % 4 != 0 || !make_row_teams(g, V, &rt, lng && NDIM == 2 ? &sg : nullptr)) return false;
+    // the plain kernel loads x in aligned groups of four voxels; the LONG one from any address
+    if (lng ? g.W < 4 : (g.W % 4 != 0 || !rows_aligned(x, g.W, 4))) return false;
+    if (!make_row_teams(g, V, &rt, lng && NDIM == 2 ? &sg : nullptr)) return false;
     if (rt.lpr % kWave != 0 || rt.lpr * rt.rpw > kThreads) return false;
-    return rows_aligned(x, g.W, 4) && rows_aligned(gy, g.W, V) && rows_aligned(gx, g.W, V);
+    return rows_aligned(gy, g.W, V) && rows_aligned(gx, g.W, V);
 }
 
 template <int NDIM>

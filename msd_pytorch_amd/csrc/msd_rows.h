@@ -39,9 +39,9 @@ struct RowSegments {
 
 constexpr int kSegmentLanes = 256;   // lanes of a team that owns a segment of a long row
 
-// With `sg`: rows longer than kSegmentLanes * V voxels are cut into segments of that length,
-// one team (and workgroup) each; the kernels that ask for it stage a halo of `dil` values on
-// either side (stage_source_segment).  2D only, whole segments only, dil <= 128.
+// With `sg`: rows longer than kSegmentLanes * V voxels are cut into segments of that length
+// (the last one may be shorter), one team (and workgroup) each; the kernels that ask for it
+// stage a halo of `dil` values on either side (stage_source_segment).  2D only, dil <= 128.
 inline bool make_row_teams(const Geom &g, int V, RowTeams *rt, RowSegments *sg = nullptr)
 {
     const int need = (g.W + V - 1) / V;
@@ -57,10 +57,10 @@ inline bool make_row_teams(const Geom &g, int V, RowTeams *rt, RowSegments *sg =
     if (sg) *sg = RowSegments{1, 0};
     if (sg && lpr > kSegmentLanes) {
         const int segw = kSegmentLanes * V;
-        if (g.ndim != 2 || g.W % segw != 0 || 2 * g.dil > kSegmentLanes) return false;
+        if (g.ndim != 2 || 2 * g.dil > kSegmentLanes) return false;
         rt->lpr = kSegmentLanes;
         rt->rpw = 1;
-        sg->segs = g.W / segw;
+        sg->segs = (g.W + segw - 1) / segw;
         sg->halo = (2 * g.dil + 3) & ~3;         // keeps what follows the staged rows 16-byte aligned
         return true;
     }
@@ -101,6 +101,16 @@ __device__ __forceinline__ void load_global_vec(uint64_t base, uint32_t byte_off
 #pragma unroll
         for (int i = 0; i < V; i++) d[i] = v[i];
     }
+}
+// Four consecutive floats at an address that is only known to be a multiple of four bytes.
+__device__ __forceinline__ void load_global_vec4_unaligned(uint64_t base, uint32_t byte_offset, float (&d)[4])
+{
+    typedef float vec_t __attribute__((ext_vector_type(4), aligned(4)));
+    typedef const __attribute__((address_space(1))) char *gbytes_t;
+    gbytes_t p = reinterpret_cast<gbytes_t>(base) + byte_offset;
+    const vec_t v = *reinterpret_cast<const __attribute__((address_space(1))) vec_t *>(p);
+#pragma unroll
+    for (int i = 0; i < 4; i++) d[i] = v[i];
 }
 template <int V>
 __device__ __forceinline__ void store_global_vec(uint64_t base, uint32_t byte_offset, const float (&d)[V])
@@ -228,7 +238,8 @@ __device__ __forceinline__ void stage_source_segment(const Geom &g, const RowTea
 {
     const AxisSources sy = adjoint_sources(y, g.H, g.dil);
     const int rs = V * rt.lpr + sg.halo;         // floats per staged row
-    const int x0 = xs + lane * V;
+    const bool inrow = rowok && xs + lane * V < g.W;   // lanes past the row stage zeros ...
+    const int x0 = min(xs + lane * V, g.W - V);        // ... read from a valid address
     const int h = lane;                          // halo element of this lane, if any
     const int hx = h < g.dil ? xs - g.dil + h : xs + V * rt.lpr + (h - g.dil);
     const bool hin = h < 2 * g.dil && hx >= 0 && hx < g.W;
@@ -245,7 +256,7 @@ __device__ __forceinline__ void stage_source_segment(const Geom &g, const RowTea
             load_vec<V>(rowp + x0, m);
             const float mh = rowp[hxc];
 #pragma unroll
-            for (int i = 0; i < V; i++) s[q][i] = (first ? 0.f : s[q][i]) + (ok && rowok ? m[i] : 0.f);
+            for (int i = 0; i < V; i++) s[q][i] = (first ? 0.f : s[q][i]) + (ok && inrow ? m[i] : 0.f);
             sh[q] = (first ? 0.f : sh[q]) + (ok && rowok && hin ? mh : 0.f);
         };
 #pragma unroll

@@ -181,6 +181,14 @@ SHAPES_XKB = [
     (1, 2, 1, (140, 2048), 129),      # dilation past that: the separate kernels
     (1, 5, 2, (8, 1024), 7),          # two output channels: 2 segments of 512
     (1, 3, 2, (4, 2048), 3),          # two output channels: 4 segments
+    # rows that are not whole groups of four voxels (unaligned rows of the input stack)
+    (1, 3, 1, (6, 750), 2),           # 2 voxels per lane, a short second segment
+    (2, 18, 1, (5, 1001), 3),         # odd: one voxel per lane, 4 segments
+    (1, 3, 1, (8, 1025), 5),          # the last segment holds one voxel: its mirrored taps come from the halo
+    (1, 5, 2, (7, 1022), 4),          # two output channels
+    (1, 4, 1, (9, 250), 3),           # whole rows per team, the last group of four is half empty
+    (1, 7, 1, (5, 6, 130), 2),        # 3D
+    (1, 3, 1, (4, 5, 127), 1),        # 3D, odd
 ]
 
 
