@@ -65,7 +65,7 @@ struct Args {
     Plane gx;            // grad_input channels (written through a cast)
     int mask_from;       // activations (viewed like grad_input) mask the channels >= mask_from
     int want_bias;
-    RowSegments sg;      // LONG instances, 2D
+    RowSegments sg;      // LONG instances
 };
 
 // Workgroups (of four waves) that are resident per CU: the 3D kernel with one voxel per lane
@@ -80,8 +80,9 @@ template <int NDIM, int V, int NCB, int WOUT> constexpr int resident_per_cu()
 
 // LONG: the variant for what the plain kernel's 32-bit lane offsets and whole-row teams do
 // not reach.  The first channel of each block of 16 moves into the uniform base of the x
-// loads (so the stack may be of any size), and 2D rows longer than a workgroup covers are cut
-// into segments, staged with a halo of `dil` values on either side.  It is a separate
+// loads (so the stack may be of any size and its rows need not be aligned or whole groups of four
+// voxels), and rows longer than a workgroup covers are cut into segments, staged with a halo of
+// `dil` values on either side.  It is a separate
 // instance because even its few extra scalar instructions per stage cost the plain one 1-4 %.
 template <int NDIM, int V, int NCB, int WOUT, bool LONG>
 __global__ __launch_bounds__(kThreads, (resident_per_cu<NDIM, V, NCB, WOUT>()))
@@ -110,7 +111,7 @@ void bwd_rows_fused(const Args a, const float *__restrict__ gyp, const float *__
     const int mk = wl / 16, mj = wl % 16;         // MFMA k (voxel group) and i/j (tap or channel) of this lane
     const int team = tid / rt.lpr, lane = tid % rt.lpr;
     // segments (rt.segs > 1): a tile is one segment of one row
-    constexpr bool SEG = LONG && NDIM == 2;
+    constexpr bool SEG = LONG;
     const bool segmented = SEG && a.sg.segs > 1;  // uniform
     const int rs = V * rt.lpr + (SEG ? a.sg.halo : 0);   // floats per staged row
     float *S = lds + (size_t)team * WOUT * NPQ * rs;
@@ -223,7 +224,7 @@ void bwd_rows_fused(const Args a, const float *__restrict__ gyp, const float *__
             const View<const float> gyv{gyp, a.gy.sb, a.gy.sc, a.gy.sz, a.gy.sy, 1};
             float own[WOUT][NPQ][V];
             if (segmented) {
-                if constexpr (SEG) stage_source_segment<WOUT, V>(g, rt, a.sg, gyv, b, yc, xs, lane, rowok, S, own);
+                if constexpr (SEG) stage_source_segment<NDIM, WOUT, V>(g, rt, a.sg, gyv, b, zc, yc, xs, lane, rowok, S, own);
             } else {
                 stage_source_rows<NDIM, false, WOUT, V>(g, rt, none, gyv, b, zc, yc, lane, act, S, own);
             }
@@ -518,7 +519,7 @@ bool fits(const Geom &g, int V, const View<const float> &gy, const View<const fl
     RowSegments sg;
     // the plain kernel loads x in aligned groups of four voxels; the LONG one from any address
     if (lng ? g.W < 4 : (g.W % 4 != 0 || !rows_aligned(x, g.W, 4))) return false;
-    if (!make_row_teams(g, V, &rt, lng && NDIM == 2 ? &sg : nullptr)) return false;
+    if (!make_row_teams(g, V, &rt, lng ? &sg : nullptr)) return false;
     if (rt.lpr % kWave != 0 || rt.lpr * rt.rpw > kThreads) return false;
     return rows_aligned(gy, g.W, V) && rows_aligned(gx, g.W, V);
 }
@@ -543,7 +544,7 @@ hipError_t launch(const Geom &g, const View<const float> &gy, const View<const f
     Args a;
     a.g = g;
     a.sg = RowSegments{1, 0};
-    make_row_teams(g, V, &a.rt, LONG && NDIM == 2 ? &a.sg : nullptr);
+    make_row_teams(g, V, &a.rt, LONG ? &a.sg : nullptr);
     // a deferred reduction brings its own region for the partial sums (defer->part)
     float *part = defer ? const_cast<float *>(defer->part) : ws + backward_k_mask_floats(g);
     a.ngroups = (a.rt.nrows + a.rt.rpw - 1) / a.rt.rpw;

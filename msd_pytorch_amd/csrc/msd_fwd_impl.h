@@ -227,15 +227,18 @@ __global__ __launch_bounds__(NDIM == 3 ? 512 : 1024, (NDIM == 3 && V == 1 && WOU
 
 constexpr size_t kMaxLds = 64 * 1024;
 
+// Threads of a workgroup (the kernel's launch bound): a row of W / V lanes must fit.
+inline int max_lanes(int ndim) { return ndim == 3 ? 512 : 1024; }
+
 inline bool make_lattice(const Geom &g, int V, int rz, int ry, int ks_wanted, Lattice *lt)
 {
     const int need = (g.W + V - 1) / V;
     const int lpr = (need + kWave - 1) / kWave * kWave;
-    if (lpr > 1024) return false;
-    int ks = ks_wanted;
     // 3D: at most 8 waves per workgroup, so that several workgroups share a CU and their
     // phases (loads, arithmetic, LDS epilogue) overlap; long rows then split less
-    const int max_threads = g.ndim == 3 ? 512 : 1024;
+    const int max_threads = max_lanes(g.ndim);
+    if (lpr > max_threads) return false;
+    int ks = ks_wanted;
     while (ks > 1 && (ks * lpr > max_threads || ks > g.C)) ks /= 2;
     if ((size_t)ks * 3 * V * lpr * sizeof(float) > kMaxLds) return false;
     lt->lpr = lpr;
@@ -285,7 +288,7 @@ inline int choose_vec(const Geom &g, int vmax, const View<const float> &x, const
         if (v > vmax) continue;
         if (!rows_aligned(x, g.W, v) || !rows_aligned(out, g.W, v)) continue;
         if (v > 1 && (g.W + v - 1) / v < kWave) continue;   // keep the lanes of a wave busy
-        if ((g.W + v - 1) / v > 1024) continue;
+        if ((g.W + v - 1) / v > max_lanes(g.ndim)) continue;
         return v;
     }
     return 0;

@@ -41,7 +41,7 @@ constexpr int kSegmentLanes = 256;   // lanes of a team that owns a segment of a
 
 // With `sg`: rows longer than kSegmentLanes * V voxels are cut into segments of that length
 // (the last one may be shorter), one team (and workgroup) each; the kernels that ask for it
-// stage a halo of `dil` values on either side (stage_source_segment).  2D only, dil <= 128.
+// stage a halo of `dil` values on either side (stage_source_segment).  dil <= 128.
 inline bool make_row_teams(const Geom &g, int V, RowTeams *rt, RowSegments *sg = nullptr)
 {
     const int need = (g.W + V - 1) / V;
@@ -57,7 +57,7 @@ inline bool make_row_teams(const Geom &g, int V, RowTeams *rt, RowSegments *sg =
     if (sg) *sg = RowSegments{1, 0};
     if (sg && lpr > kSegmentLanes) {
         const int segw = kSegmentLanes * V;
-        if (g.ndim != 2 || 2 * g.dil > kSegmentLanes) return false;
+        if (2 * g.dil > kSegmentLanes) return false;
         rt->lpr = kSegmentLanes;
         rt->rpw = 1;
         sg->segs = (g.W + segw - 1) / segw;
@@ -227,53 +227,68 @@ __device__ __forceinline__ void stage_source_rows(const Geom &g, const RowTeams 
     __syncthreads();
 }
 
-// Segment variant of stage_source_rows (2D, no ReLU mask): the team owns voxels
-// [xs, xs + V * lpr) of row y.  A staged row holds the segment in the usual layout, then
+// Segment variant of stage_source_rows (no ReLU mask): the team owns voxels
+// [xs, xs + V * lpr) of row (z, y).  A staged row holds the segment in the usual layout, then
 // `dil` values to the left of it and `dil` values to the right (zeros outside the row), which
 // the lanes 0 .. 2 dil - 1 load one each.  Ends with a workgroup barrier.
-template <int WOUT, int V>
+template <int NDIM, int WOUT, int V>
 __device__ __forceinline__ void stage_source_segment(const Geom &g, const RowTeams &rt, const RowSegments &sg,
-                                                     const View<const float> &gy, int b, int y, int xs, int lane, bool rowok,
-                                                     float *__restrict__ S, float (&own)[WOUT][3][V])
+                                                     const View<const float> &gy, int b, int z, int y, int xs,
+                                                     int lane, bool rowok, float *__restrict__ S,
+                                                     float (&own)[WOUT][RowTaps<NDIM>::NPQ][V])
 {
+    constexpr int NZ = Taps<NDIM>::NZ, NPQ = RowTaps<NDIM>::NPQ;
+    const AxisSources sz = NDIM == 3 ? adjoint_sources(z, g.D, g.dil) : single_source();
     const AxisSources sy = adjoint_sources(y, g.H, g.dil);
     const int rs = V * rt.lpr + sg.halo;         // floats per staged row
     const bool inrow = rowok && xs + lane * V < g.W;   // lanes past the row stage zeros ...
     const int x0 = min(xs + lane * V, g.W - V);        // ... read from a valid address
     const int h = lane;                          // halo element of this lane, if any
     const int hx = h < g.dil ? xs - g.dil + h : xs + V * rt.lpr + (h - g.dil);
-    const bool hin = h < 2 * g.dil && hx >= 0 && hx < g.W;
+    const bool hin = rowok && h < 2 * g.dil && hx >= 0 && hx < g.W;
     const int hxc = min(max(hx, 0), g.W - 1);
-    const bool folds = y < g.dil || y + g.dil >= g.H;
+    const bool folds = y < g.dil || y + g.dil >= g.H || (NDIM == 3 && (z < g.dil || z + g.dil >= g.D));
 #pragma unroll
     for (int co = 0; co < WOUT; co++) {
         const float *gc = gy.p + (int64_t)b * gy.sb + (int64_t)co * gy.sc;
-        float s[3][V], sh[3];
-        auto add_row = [&](int q, int cy, bool ok, bool first) {
+        float s[NPQ][V], sh[NPQ];
+        auto add_row = [&](int pq, int cz, int cy, bool ok, bool first) {
+            cz = min(max(cz, 0), g.D - 1);
             cy = min(max(cy, 0), g.H - 1);
-            const float *rowp = gc + (int64_t)cy * gy.sy;
+            const float *rowp = gc + (int64_t)cz * gy.sz + (int64_t)cy * gy.sy;
             float m[V];
             load_vec<V>(rowp + x0, m);
             const float mh = rowp[hxc];
 #pragma unroll
-            for (int i = 0; i < V; i++) s[q][i] = (first ? 0.f : s[q][i]) + (ok && inrow ? m[i] : 0.f);
-            sh[q] = (first ? 0.f : sh[q]) + (ok && rowok && hin ? mh : 0.f);
+            for (int i = 0; i < V; i++) s[pq][i] = (first ? 0.f : s[pq][i]) + (ok && inrow ? m[i] : 0.f);
+            sh[pq] = (first ? 0.f : sh[pq]) + (ok && hin ? mh : 0.f);
         };
 #pragma unroll
-        for (int q = 0; q < 3; q++) add_row(q, sy.c[q][0], sy.ok[q][0], true);
+        for (int p = 0; p < NZ; p++)
+#pragma unroll
+            for (int q = 0; q < 3; q++)
+                add_row(p * 3 + q, sz.c[p][0], sy.c[q][0], sz.ok[p][0] && sy.ok[q][0], true);
         if (folds) {
 #pragma unroll
-            for (int q = 0; q < 3; q++) add_row(q, sy.c[q][1], sy.ok[q][1], false);
+            for (int p = 0; p < NZ; p++)
+#pragma unroll
+                for (int q = 0; q < 3; q++) {
+                    add_row(p * 3 + q, sz.c[p][0], sy.c[q][1], sz.ok[p][0] && sy.ok[q][1], false);
+                    if (NDIM == 3) {
+                        add_row(p * 3 + q, sz.c[p][1], sy.c[q][0], sz.ok[p][1] && sy.ok[q][0], false);
+                        add_row(p * 3 + q, sz.c[p][1], sy.c[q][1], sz.ok[p][1] && sy.ok[q][1], false);
+                    }
+                }
         }
 #pragma unroll
-        for (int q = 0; q < 3; q++) {
-            float *row = S + (size_t)(co * 3 + q) * rs;
+        for (int pq = 0; pq < NPQ; pq++) {
+            float *row = S + (size_t)(co * NPQ + pq) * rs;
 #pragma unroll
             for (int i = 0; i < V; i++) {
-                own[co][q][i] = s[q][i];
-                row[i * rt.lpr + lane] = s[q][i];
+                own[co][pq][i] = s[pq][i];
+                row[i * rt.lpr + lane] = s[pq][i];
             }
-            if (h < 2 * g.dil) row[V * rt.lpr + h] = sh[q];
+            if (h < 2 * g.dil) row[V * rt.lpr + h] = sh[pq];
         }
     }
     __syncthreads();

@@ -34,6 +34,9 @@ SHAPES_FAST = [
     (1, 6, 1, (20, 21, 70), 3),
     (2, 4, 2, (12, 33, 65), 2),
     (1, 9, 1, (32, 32, 128), 10),
+    (1, 3, 1, (3, 5, 600), 2),       # 3D rows longer than the forward kernel's 512 lanes: 4 voxels per lane
+    (1, 2, 1, (2, 4, 601), 1),       # the same, odd: shape-generic forward
+    (1, 2, 2, (3, 2100), 3),         # 2D, long ragged rows, two output channels
 ]
 
 

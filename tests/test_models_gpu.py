@@ -75,6 +75,7 @@ FUSED_BLOCK_CASES = [
     (2, (11, 750), 1, 4, 1, None),         # rows that are not whole groups of four voxels
     (2, (6, 1001), 2, 3, 2, [1, 5, 3], 2),   # odd rows, width 2
     (3, (5, 6, 130), 1, 3, 1, None),       # the same in 3D
+    (3, (4, 7, 516), 2, 3, 1, [2, 4, 1]),  # 3D rows of three segments
 ]
 
 

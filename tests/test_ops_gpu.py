@@ -189,6 +189,8 @@ SHAPES_XKB = [
     (1, 4, 1, (9, 250), 3),           # whole rows per team, the last group of four is half empty
     (1, 7, 1, (5, 6, 130), 2),        # 3D
     (1, 3, 1, (4, 5, 127), 1),        # 3D, odd
+    (1, 3, 1, (4, 5, 512), 3),        # 3D rows of two segments
+    (2, 18, 1, (3, 4, 300), 2),       # 3D, a short second segment, folds in z and y
 ]
 
 

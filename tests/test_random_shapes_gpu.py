@@ -19,7 +19,7 @@ def _random_shape(rng, ndim):
     if ndim == 2:
         size = (rng.randrange(1, 48), w)
     else:
-        w = min(w, 260)
+        w = min(w, rng.choice([260, 260, 600]))
         size = (rng.randrange(1, 12), rng.randrange(1, 14), w)
     d = rng.randrange(1, min(min(size), 10) + 1)
     c_in = rng.choice([1, 2, 3, 7, 15, 16, 17, 31, 32, 33, 40])
