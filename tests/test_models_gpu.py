@@ -186,6 +186,31 @@ def test_single_layer_gradcheck_f64(ndim, size):
         assert torch.autograd.gradcheck(f, (x, w, b), eps=1e-6, atol=1e-5)
 
 
+def test_module_rejects_zero_depth_and_width():
+    # tests/test_msd_module.py:133-137 of the reference
+    from msd_pytorch_amd import MSDModule
+    with pytest.raises(ValueError):
+        MSDModule(1, 1, depth=0, width=1)
+    with pytest.raises(ValueError):
+        MSDModule(1, 1, depth=1, width=0)
+
+
+@pytest.mark.parametrize("mean", [-10, 0, 10])
+@pytest.mark.parametrize("std", [1, 10])
+def test_normalization_scale_out_inverts_scale_in(mean, std):
+    # tests/test_msd_model.py:6-36 of the reference: input and target with the same moments make
+    # the two frozen scaling layers each other's inverse
+    from msd_pytorch_amd.msd_model import MSDModel
+    from torch.utils.data import DataLoader, TensorDataset
+    torch.manual_seed(1)
+    model = MSDModel(3, 3, 10, 1)
+    d_in = mean + torch.randn(1, 3, 100, 100) * std
+    model.set_normalization(DataLoader(TensorDataset(d_in, d_in.clone()), 1))
+    x = torch.randn_like(d_in).cuda()
+    y = model.scale_out.cuda()(model.scale_in.cuda()(x))
+    assert (x - y).abs().mean().item() < 1e-4
+
+
 def test_module_zero_output_then_all_parameters_move():
     # reference tests/test_msd_module.py:11-16 and :87-130
     from msd_pytorch_amd.msd_module import MSDModule
