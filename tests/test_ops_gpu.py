@@ -229,3 +229,54 @@ def test_backward_xkb_without_bias_and_errors(cc):
         cc.conv_backward_xkb(p["gy"], p["x"], p["k"], p["gx"], gk, None, 65)      # dilation > size
     with pytest.raises(RuntimeError):
         cc.conv_backward_xkb(p["gy"].cpu(), p["x"], p["k"], p["gx"], gk, None, 1)  # CPU tensor
+
+
+# The reference's own value tests (tests/test_conv2d.py:126-186, tests/test_conv3d.py:323-374):
+# away from the borders symmetric padding plays no part, so the centre of the output must
+# agree with torch's zero-padded dilated convolution.  Their parameter grid, in double; torch's
+# convolution runs on the CPU (an independent implementation, no GPU library involved).
+REFERENCE_VALUE_GRID = [(2, 3, 5, d, size) for d in (1, 3, 10) for size in (2 * d + 1, 29, 50)]
+
+
+@pytest.mark.parametrize("ndim", [2, 3])
+@pytest.mark.parametrize("B,c_in,c_out,d,size", REFERENCE_VALUE_GRID)
+def test_centre_agrees_with_torch_convolution(ndim, B, c_in, c_out, d, size):
+    import torch.nn.functional as F
+    from msd_pytorch_amd.conv2d import conv2d_forward
+    from msd_pytorch_amd.conv3d import conv3d_relu
+    shape = (size, 2 * size) if ndim == 2 else (size, 2 * size, 3 * size)
+    gen = torch.Generator().manual_seed(d * 100 + size)
+    x = torch.randn(B, c_in, *shape, dtype=torch.double, generator=gen)
+    k = torch.randn(c_out, c_in, *([3] * ndim), dtype=torch.double, generator=gen)
+    bias = torch.randn(c_out, dtype=torch.double, generator=gen)
+    y = torch.zeros(B, c_out, *shape, dtype=torch.double, device="cuda")
+    if ndim == 2:
+        conv2d_forward(x.cuda(), k.cuda(), bias.cuda(), y, d)
+        want = F.conv2d(x, k, bias, padding=d, dilation=d)
+    else:
+        conv3d_relu(x.cuda(), k.cuda(), bias.cuda(), y, 1, d)
+        want = F.relu(F.conv3d(x, k, bias, padding=d, dilation=d))
+    assert want.shape == y.shape
+    centre = (slice(None), slice(None)) + (slice(d, -d),) * ndim
+    assert torch.allclose(y.cpu()[centre], want[centre], rtol=1e-10, atol=1e-10)
+
+
+@pytest.mark.parametrize("ndim,size", [(2, 128), (3, 44)])
+@pytest.mark.parametrize("c_out", [1, 2])
+@pytest.mark.parametrize("d", [1, 4, 10])
+def test_centre_agrees_with_torch_convolution_f32_specialised(ndim, size, c_out, d):
+    # the same check at shapes the specialised fp32 kernels take (rows of 256 / 132 voxels,
+    # one or two output channels); tolerance: forward, relative 1e-5
+    import torch.nn.functional as F
+    shape = (size, 2 * size) if ndim == 2 else (size, size + 3, 3 * size)
+    gen = torch.Generator().manual_seed(d)
+    x = torch.randn(2, 7, *shape, generator=gen)
+    k = torch.randn(c_out, 7, *([3] * ndim), generator=gen) * 0.2
+    bias = torch.randn(c_out, generator=gen)
+    y = torch.zeros(2, c_out, *shape, device="cuda")
+    from msd_pytorch_amd import msd_custom_convolutions as native
+    native.conv_relu_forward(x.cuda(), k.cuda(), bias.cuda(), y, d)
+    conv = F.conv2d if ndim == 2 else F.conv3d
+    want = F.relu(conv(x.double(), k.double(), bias.double(), padding=d, dilation=d))
+    centre = (slice(None), slice(None)) + (slice(d, -d),) * ndim
+    assert rel_err(y.cpu()[centre], want[centre]) <= 1e-5
