@@ -48,7 +48,37 @@ def _wide_cases(seed, n):
     return out
 
 
-@pytest.mark.parametrize("shape", _cases(2024, 40) + _wide_cases(77, 10), ids=lambda s: "B%d-C%d-w%d-%s-d%d" % (
+def _extreme_cases(seed, n):
+    # the corners: rows of 1 to 8192 voxels (beyond every kernel's row limit), flat images,
+    # channel counts around the chunks of 128, dilations up to the smallest extent and around
+    # the halo limit, layers of up to five output channels, batches of five
+    rng = random.Random(seed)
+    out = []
+    for _ in range(n):
+        ndim = rng.choice([2, 2, 3])
+        if ndim == 2:
+            w = rng.choice([1, 2, 3, 5, 31, 33, 63, 65, 255, 257, 1023, 1025, 4096, 4100, 5000, 8192,
+                            rng.randrange(1, 6000)])
+            h = rng.choice([1, 2, 3, rng.randrange(1, 40), rng.randrange(100, 300)])
+            if w * h > 600000:
+                h = max(1, 600000 // w)
+            size = (h, w)
+        else:
+            w = rng.choice([1, 2, 31, 33, 65, 255, 257, 511, 513, 520, 1024, 1030, 2048, rng.randrange(1, 1200)])
+            a, b = rng.choice([1, 2, 3, rng.randrange(1, 30)]), rng.choice([1, 2, 5, rng.randrange(1, 30)])
+            while w * a * b > 400000 and (a > 1 or b > 1):
+                a, b = max(1, a // 2), max(1, b // 2)
+            size = (a, b, w)
+        m = min(size)
+        d = max(1, rng.choice([1, m, rng.randrange(1, m + 1), min(m, 127), min(m, 129)]))
+        c_in = rng.choice([1, 2, 16, 17, 64, 65, 128, 129, 140])
+        if c_in * size[-1] * (size[0] if ndim == 2 else size[0] * size[1]) > 6e6:
+            c_in = rng.choice([1, 2, 3])
+        out.append((rng.choice([1, 2, 5]), c_in, rng.choice([1, 1, 2, 3, 5]), size, d))
+    return out
+
+
+@pytest.mark.parametrize("shape", _cases(2024, 40) + _wide_cases(77, 10) + _extreme_cases(901, 30), ids=lambda s: "B%d-C%d-w%d-%s-d%d" % (
     s[0], s[1], s[2], "x".join(map(str, s[3])), s[4]))
 def test_random_operator_problems(shape):
     from msd_pytorch_amd import msd_custom_convolutions as cc
