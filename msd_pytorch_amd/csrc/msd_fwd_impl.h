@@ -227,6 +227,12 @@ __global__ __launch_bounds__(NDIM == 3 ? 512 : 1024, (NDIM == 3 && V == 1 && WOU
 
 constexpr size_t kMaxLds = 64 * 1024;
 
+// 2D: while the input channels of a layer fit the 256 MB memory-side cache, one voxel per lane
+// (a row of 1024 lanes, 16 waves per CU) is 8-15 % faster than four (8 waves): the loads come
+// back sooner than from memory and more waves keep more of them in flight.  Past that size
+// the wider loads win by as much (1024 x 1024, 60 against 70 channels).
+constexpr int64_t kCacheResidentBytes = 256 * 1000 * 1000;
+
 // Threads of a workgroup (the kernel's launch bound): a row of W / V lanes must fit.
 inline int max_lanes(int ndim) { return ndim == 3 ? 512 : 1024; }
 
@@ -307,7 +313,10 @@ template <int NDIM, bool RELU, int WOUT>
 hipError_t pick(const Geom &g, const View<const float> &x, const float *k, const float *bias, const View<float> &out,
                 hipStream_t s)
 {
-    const int vmax = knob(NDIM == 3 ? kKnobFwdVec3d : kKnobFwdVec2d, NDIM == 3 ? 1 : 4);
+    int vmax = knob(NDIM == 3 ? kKnobFwdVec3d : kKnobFwdVec2d, NDIM == 3 ? 1 : 4);
+    if (NDIM == 2 && WOUT == 1 && knob(kKnobFwdVec2d, -1) < 0 &&
+        (int64_t)g.B * g.C * x.sc * (int64_t)sizeof(float) <= kCacheResidentBytes)
+        vmax = 1;
     int v = choose_vec(g, vmax, x, out);
     if (v == 0) v = choose_vec(g, 4, x, out);
     if constexpr (NDIM == 3) {
@@ -315,7 +324,7 @@ hipError_t pick(const Geom &g, const View<const float> &x, const float *k, const
         if (v == 2) return launch<3, RELU, WOUT, 2, 2, 4>(g, x, k, bias, out, s);
         if (v == 1) return launch<3, RELU, WOUT, 1, 2, 4>(g, x, k, bias, out, s);
     } else {
-        if (v == 4 && WOUT == 1) {
+        if constexpr (WOUT == 1) {
             // Rows per tile: all tiles cost the same, so the time is (rounds of tiles over
             // the 256 CUs) x (rows per tile); with few tiles a longer chain that avoids a
             // nearly empty last round wins.
@@ -327,16 +336,27 @@ hipError_t pick(const Geom &g, const View<const float> &x, const float *k, const
                 if (ry == 4 || cost < best_cost) { best = ry; best_cost = cost; }
             }
             best = knob(kKnobFwdRows2d, best);
-            if (best == 5) return launch<2, RELU, 1, 4, 1, 5>(g, x, k, bias, out, s);
-            if (best == 6) return launch<2, RELU, 1, 4, 1, 6>(g, x, k, bias, out, s);
+            if (v == 4) {
+                if (best == 5) return launch<2, RELU, 1, 4, 1, 5>(g, x, k, bias, out, s);
+                if (best == 6) return launch<2, RELU, 1, 4, 1, 6>(g, x, k, bias, out, s);
+                return launch<2, RELU, 1, 4, 1, 4>(g, x, k, bias, out, s);
+            }
+            if (v == 2) {
+                if (best == 5) return launch<2, RELU, 1, 2, 1, 5>(g, x, k, bias, out, s);
+                if (best == 6) return launch<2, RELU, 1, 2, 1, 6>(g, x, k, bias, out, s);
+                return launch<2, RELU, 1, 2, 1, 4>(g, x, k, bias, out, s);
+            }
+            if (v == 1) {
+                if (best == 5) return launch<2, RELU, 1, 1, 1, 5>(g, x, k, bias, out, s);
+                if (best == 6) return launch<2, RELU, 1, 1, 1, 6>(g, x, k, bias, out, s);
+                return launch<2, RELU, 1, 1, 1, 4>(g, x, k, bias, out, s);
+            }
+        } else {
+            // two output channels double the accumulators: three rows per tile keep them in registers
+            if (v == 4) return launch<2, RELU, 2, 4, 1, 3>(g, x, k, bias, out, s);
+            if (v == 2) return launch<2, RELU, 2, 2, 1, 4>(g, x, k, bias, out, s);
+            if (v == 1) return launch<2, RELU, 2, 1, 1, 4>(g, x, k, bias, out, s);
         }
-        // two output channels double the accumulators: three rows per tile keep them in registers
-        if (v == 4 && WOUT == 2) return launch<2, RELU, 2, 4, 1, 3>(g, x, k, bias, out, s);
-        if constexpr (WOUT == 1) {
-            if (v == 4) return launch<2, RELU, 1, 4, 1, 4>(g, x, k, bias, out, s);
-        }
-        if (v == 2) return launch<2, RELU, WOUT, 2, 1, 4>(g, x, k, bias, out, s);
-        if (v == 1) return launch<2, RELU, WOUT, 1, 1, 4>(g, x, k, bias, out, s);
     }
     return hipErrorInvalidConfiguration;
 }
