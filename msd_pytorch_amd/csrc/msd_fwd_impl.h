@@ -314,9 +314,8 @@ hipError_t pick(const Geom &g, const View<const float> &x, const float *k, const
                 hipStream_t s)
 {
     int vmax = knob(NDIM == 3 ? kKnobFwdVec3d : kKnobFwdVec2d, NDIM == 3 ? 1 : 4);
-    if (NDIM == 2 && WOUT == 1 && knob(kKnobFwdVec2d, -1) < 0 &&
-        (int64_t)g.B * g.C * x.sc * (int64_t)sizeof(float) <= kCacheResidentBytes)
-        vmax = 1;
+    const bool resident = (int64_t)g.B * g.C * x.sc * (int64_t)sizeof(float) <= kCacheResidentBytes;
+    if (NDIM == 2 && WOUT == 1 && knob(kKnobFwdVec2d, -1) < 0 && resident) vmax = 1;
     int v = choose_vec(g, vmax, x, out);
     if (v == 0) v = choose_vec(g, 4, x, out);
     if constexpr (NDIM == 3) {
@@ -327,26 +326,37 @@ hipError_t pick(const Geom &g, const View<const float> &x, const float *k, const
         if constexpr (WOUT == 1) {
             // Rows per tile: all tiles cost the same, so the time is (rounds of tiles over
             // the 256 CUs) x (rows per tile); with few tiles a longer chain that avoids a
-            // nearly empty last round wins.
-            int best = 4;
+            // nearly empty last round wins.  Tiles of 2 or 3 rows read 2 and 1.67 input rows
+            // per output row instead of 1.5 and less: they are candidates only for images so
+            // small that tiles of four rows leave CUs idle, and while the input comes from
+            // the cache (256 x 256, 100 channels: 16 against 21 us).
+            const long tiles4 = (long)g.dil * (((g.H + g.dil - 1) / g.dil + 3) / 4) * g.B;
+            const int first = resident && tiles4 < 256 ? 2 : 4;
+            int best = first;
             long best_cost = 0;
-            for (int ry = 4; ry <= 6; ry++) {
+            for (int ry = first; ry <= 6; ry++) {
                 const long tiles = (long)g.dil * (((g.H + g.dil - 1) / g.dil + ry - 1) / ry) * g.B;
                 const long cost = (tiles + 255) / 256 * ry;
-                if (ry == 4 || cost < best_cost) { best = ry; best_cost = cost; }
+                if (ry == first || cost < best_cost) { best = ry; best_cost = cost; }
             }
             best = knob(kKnobFwdRows2d, best);
             if (v == 4) {
+                if (best == 2) return launch<2, RELU, 1, 4, 1, 2>(g, x, k, bias, out, s);
+                if (best == 3) return launch<2, RELU, 1, 4, 1, 3>(g, x, k, bias, out, s);
                 if (best == 5) return launch<2, RELU, 1, 4, 1, 5>(g, x, k, bias, out, s);
                 if (best == 6) return launch<2, RELU, 1, 4, 1, 6>(g, x, k, bias, out, s);
                 return launch<2, RELU, 1, 4, 1, 4>(g, x, k, bias, out, s);
             }
             if (v == 2) {
+                if (best == 2) return launch<2, RELU, 1, 2, 1, 2>(g, x, k, bias, out, s);
+                if (best == 3) return launch<2, RELU, 1, 2, 1, 3>(g, x, k, bias, out, s);
                 if (best == 5) return launch<2, RELU, 1, 2, 1, 5>(g, x, k, bias, out, s);
                 if (best == 6) return launch<2, RELU, 1, 2, 1, 6>(g, x, k, bias, out, s);
                 return launch<2, RELU, 1, 2, 1, 4>(g, x, k, bias, out, s);
             }
             if (v == 1) {
+                if (best == 2) return launch<2, RELU, 1, 1, 1, 2>(g, x, k, bias, out, s);
+                if (best == 3) return launch<2, RELU, 1, 1, 1, 3>(g, x, k, bias, out, s);
                 if (best == 5) return launch<2, RELU, 1, 1, 1, 5>(g, x, k, bias, out, s);
                 if (best == 6) return launch<2, RELU, 1, 1, 1, 6>(g, x, k, bias, out, s);
                 return launch<2, RELU, 1, 1, 1, 4>(g, x, k, bias, out, s);
