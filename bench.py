@@ -29,8 +29,8 @@ HBM_PEAK_GBS = 8000.0
 # WRITE_SIZE x 1.000).  Counters cannot be read from inside this script, so the figures
 # of the committed profiles are carried here; a class without one reports null.
 TRAFFIC = {
-    "C": {"forward": 22.218e9, "backward_xkb": 65.041e9 + 0.096e9},
-    "D": {"forward": 16.252e9, "backward_xkb": 34.596e9 + 0.072e9},
+    "C": {"forward": 22.191e9, "backward_xkb": 65.040e9 + 0.096e9},
+    "D": {"forward": 16.248e9, "backward_xkb": 34.596e9 + 0.072e9},
 }
 
 WORKLOADS = {
