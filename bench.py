@@ -32,7 +32,7 @@ TRAFFIC = {
     "C": {"forward": 22.191e9, "backward_xkb": 65.040e9 + 0.096e9},
     "D": {"forward": 16.248e9, "backward_xkb": 34.596e9 + 0.072e9},
     "E1": {"forward": 763.269e9, "backward_xkb": 2121.959e9 + 1.514e9},
-    "E2": {"forward": 53.120e9, "backward_xkb": 101.806e9 + 0.095e9},
+    "E2": {"forward": 53.120e9, "backward_xkb": 101.806e9 + 0.039e9},
 }
 
 WORKLOADS = {
