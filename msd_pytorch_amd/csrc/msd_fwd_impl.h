@@ -321,7 +321,19 @@ hipError_t pick(const Geom &g, const View<const float> &x, const float *k, const
     if constexpr (NDIM == 3) {
         if (v == 4) return launch<3, RELU, WOUT, 4, 2, 2>(g, x, k, bias, out, s);
         if (v == 2) return launch<3, RELU, WOUT, 2, 2, 4>(g, x, k, bias, out, s);
-        if (v == 1) return launch<3, RELU, WOUT, 1, 2, 4>(g, x, k, bias, out, s);
+        if (v == 1) {
+            if constexpr (WOUT == 1) {
+                // Lattices of 3 x 3 rows instead of 2 x 4 where they cover the residue classes
+                // with at least 1/16 fewer tiles (a partly filled lattice costs as much time as a
+                // full one): at 128^3 dilations 3, 5, 9, 10, by 2 to 12 %.  Not at dilations 1
+                // and 2, where the nine rows per tile cost more than the fewer tiles save.
+                const int rows_y = (g.H + g.dil - 1) / g.dil, rows_z = (g.D + g.dil - 1) / g.dil;
+                const long t24 = (long)((rows_z + 1) / 2) * ((rows_y + 3) / 4);
+                const long t33 = (long)((rows_z + 2) / 3) * ((rows_y + 2) / 3);
+                if (g.dil >= 3 && t33 * 16 < t24 * 15) return launch<3, RELU, 1, 1, 3, 3>(g, x, k, bias, out, s);
+            }
+            return launch<3, RELU, WOUT, 1, 2, 4>(g, x, k, bias, out, s);
+        }
     } else {
         if constexpr (WOUT == 1) {
             // Rows per tile: all tiles cost the same, so the time is (rounds of tiles over
