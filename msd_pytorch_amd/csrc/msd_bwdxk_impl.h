@@ -634,7 +634,22 @@ hipError_t xkb_nd(const Geom &g, const View<const float> &gy, const View<const f
                   ReduceJob *defer)
 {
     // 3D: one voxel per lane keeps the 27 gathered values per voxel and the pipeline buffers in registers
-    const int vmax = knob(NDIM == 3 ? kKnobBwdkVec3d : kKnobBwdkVec2d, NDIM == 3 ? 1 : 4);
+    int vmax = knob(NDIM == 3 ? kKnobBwdkVec3d : kKnobBwdkVec2d, NDIM == 3 ? 1 : 4);
+    if (NDIM == 2 && !LONG && knob(kKnobBwdkVec2d, -1) < 0) {
+        // Small images: fewer voxels per lane make more tiles (a tile is 256 lanes: one long row or
+        // several short ones).  The widest vector that still fills the 512 resident workgroups
+        // wins, else the one with the most tiles (256 x 256, 100 channels: 58 -> 39 us).
+        int best = 0;
+        int64_t best_tiles = 0;
+        for (int v = g.Wd == 2 ? kMaxVecTwoOutputs : 4; v >= 1; v /= 2) {
+            RowTeams rt;
+            if (!fits<NDIM>(g, v, gy, x, gx, LONG) || !make_row_teams(g, v, &rt)) continue;
+            const int64_t tiles = (int64_t)g.B * ((rt.nrows + rt.rpw - 1) / rt.rpw);
+            if (tiles > best_tiles) { best = v; best_tiles = tiles; }
+            if (tiles >= 512) break;
+        }
+        if (best) vmax = best;
+    }
     int v = choose_vec<NDIM>(g, vmax, gy, x, gx, LONG);
     if (v == 0) v = choose_vec<NDIM>(g, 4, gy, x, gx, LONG);
     if constexpr (NDIM == 2) {
