@@ -29,8 +29,8 @@ HBM_PEAK_GBS = 8000.0
 # WRITE_SIZE x 1.000).  Counters cannot be read from inside this script, so the figures
 # of the committed profiles are carried here; a class without one reports null.
 TRAFFIC = {
-    "C": {"forward": 22.191e9, "backward_xkb": 65.040e9 + 0.096e9},
-    "D": {"forward": 16.248e9, "backward_xkb": 34.596e9 + 0.072e9},
+    "C": {"forward": 22.187e9, "backward_xkb": 65.038e9 + 0.096e9},
+    "D": {"forward": 16.151e9, "backward_xkb": 34.598e9 + 0.072e9},
     "E1": {"forward": 763.269e9, "backward_xkb": 2121.959e9 + 1.514e9},
     "E2": {"forward": 53.120e9, "backward_xkb": 101.806e9 + 0.039e9},
 }
