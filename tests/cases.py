@@ -37,6 +37,9 @@ SHAPES_FAST = [
     (1, 3, 1, (3, 5, 600), 2),       # 3D rows longer than the forward kernel's 512 lanes: 4 voxels per lane
     (1, 2, 1, (2, 4, 601), 1),       # the same, odd: shape-generic forward
     (1, 2, 2, (3, 2100), 3),         # 2D, long ragged rows, two output channels
+    (1, 5, 3, (40, 132), 2),         # three output channels: the specialised kernels in groups of 2 + 1
+    (2, 4, 5, (9, 12, 68), 3),       # 3D, five output channels: 2 + 2 + 1
+    (1, 3, 4, (6, 1022), 4),         # four output channels, rows of 2 voxels per lane
 ]
 
 

@@ -76,6 +76,8 @@ FUSED_BLOCK_CASES = [
     (2, (6, 1001), 2, 3, 2, [1, 5, 3], 2),   # odd rows, width 2
     (3, (5, 6, 130), 1, 3, 1, None),       # the same in 3D
     (3, (4, 7, 516), 2, 3, 1, [2, 4, 1]),  # 3D rows of three segments
+    (2, (30, 132), 2, 4, 1, None, 3),      # width 3: the separate kernels, two output channels at a time
+    (3, (6, 7, 68), 1, 3, 2, None, 3),     # the same in 3D
 ]
 
 
