@@ -309,6 +309,20 @@ bool supported_nd(const Geom &g, const View<const float> &x, const View<float> &
     return choose_vec(g, 4, x, out) != 0;
 }
 
+// 2D, one output channel: the instance with `ry` output rows per tile (2 to 6; 4 otherwise).
+template <bool RELU, int V>
+hipError_t launch_rows_2d(int ry, const Geom &g, const View<const float> &x, const float *k, const float *bias,
+                          const View<float> &out, hipStream_t s)
+{
+    switch (ry) {
+    case 2: return launch<2, RELU, 1, V, 1, 2>(g, x, k, bias, out, s);
+    case 3: return launch<2, RELU, 1, V, 1, 3>(g, x, k, bias, out, s);
+    case 5: return launch<2, RELU, 1, V, 1, 5>(g, x, k, bias, out, s);
+    case 6: return launch<2, RELU, 1, V, 1, 6>(g, x, k, bias, out, s);
+    default: return launch<2, RELU, 1, V, 1, 4>(g, x, k, bias, out, s);
+    }
+}
+
 template <int NDIM, bool RELU, int WOUT>
 hipError_t pick(const Geom &g, const View<const float> &x, const float *k, const float *bias, const View<float> &out,
                 hipStream_t s)
@@ -352,27 +366,9 @@ hipError_t pick(const Geom &g, const View<const float> &x, const float *k, const
                 if (ry == first || cost < best_cost) { best = ry; best_cost = cost; }
             }
             best = knob(kKnobFwdRows2d, best);
-            if (v == 4) {
-                if (best == 2) return launch<2, RELU, 1, 4, 1, 2>(g, x, k, bias, out, s);
-                if (best == 3) return launch<2, RELU, 1, 4, 1, 3>(g, x, k, bias, out, s);
-                if (best == 5) return launch<2, RELU, 1, 4, 1, 5>(g, x, k, bias, out, s);
-                if (best == 6) return launch<2, RELU, 1, 4, 1, 6>(g, x, k, bias, out, s);
-                return launch<2, RELU, 1, 4, 1, 4>(g, x, k, bias, out, s);
-            }
-            if (v == 2) {
-                if (best == 2) return launch<2, RELU, 1, 2, 1, 2>(g, x, k, bias, out, s);
-                if (best == 3) return launch<2, RELU, 1, 2, 1, 3>(g, x, k, bias, out, s);
-                if (best == 5) return launch<2, RELU, 1, 2, 1, 5>(g, x, k, bias, out, s);
-                if (best == 6) return launch<2, RELU, 1, 2, 1, 6>(g, x, k, bias, out, s);
-                return launch<2, RELU, 1, 2, 1, 4>(g, x, k, bias, out, s);
-            }
-            if (v == 1) {
-                if (best == 2) return launch<2, RELU, 1, 1, 1, 2>(g, x, k, bias, out, s);
-                if (best == 3) return launch<2, RELU, 1, 1, 1, 3>(g, x, k, bias, out, s);
-                if (best == 5) return launch<2, RELU, 1, 1, 1, 5>(g, x, k, bias, out, s);
-                if (best == 6) return launch<2, RELU, 1, 1, 1, 6>(g, x, k, bias, out, s);
-                return launch<2, RELU, 1, 1, 1, 4>(g, x, k, bias, out, s);
-            }
+            if (v == 4) return launch_rows_2d<RELU, 4>(best, g, x, k, bias, out, s);
+            if (v == 2) return launch_rows_2d<RELU, 2>(best, g, x, k, bias, out, s);
+            if (v == 1) return launch_rows_2d<RELU, 1>(best, g, x, k, bias, out, s);
         } else {
             // two output channels double the accumulators: three rows per tile keep them in registers
             if (v == 4) return launch<2, RELU, 2, 4, 1, 3>(g, x, k, bias, out, s);
