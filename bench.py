@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Headline benchmark: MSD train step (forward + backward) on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C|D|A|B|E2]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C|D|A|B|E1|E2]
 
 Prints ONE JSON line.  `value` is megavoxels per second of one training step
 (batch * voxels / step time) of the workload, inputs resident in HBM.  The
@@ -22,18 +22,48 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# fp32 peak of MI355X (matrix cores, or packed vector instructions); plain (non-packed) vector
+# fp32, which the build rules leave to the forward kernel's multiply-adds, peaks at half of it
+FP32_PEAK_TFLOPS = 157.3
+PIPE = {"forward": "fp32 VALU, non-packed (78.6 TFLOP/s of the 157.3 peak)",
+        "backward_x": "fp32 VALU, non-packed (78.6 TFLOP/s of the 157.3 peak)",
+        "backward_kb": "fp32 MFMA 16x16x4",
+        "backward_xkb": "fp32 MFMA 16x16x4 (weight gradient) + fp32 VALU (input gradient), half of the flops each"}
 
-# HBM-side bytes per step of each kernel class from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE (summaries and commands under profiles/), each scaled by what the same
-# counter reads for a 1 GiB device copy in the same run (FETCH_SIZE x 2.000,
-# WRITE_SIZE x 1.000).  Counters cannot be read from inside this script, so the figures
-# of the committed profiles are carried here; a class without one reports null.
-TRAFFIC = {
-    "C": {"forward": 22.187e9, "backward_xkb": 65.038e9 + 0.096e9},
-    "D": {"forward": 16.151e9, "backward_xkb": 34.598e9 + 0.072e9},
-    "E1": {"forward": 763.269e9, "backward_xkb": 2121.959e9 + 1.514e9},
-    "E2": {"forward": 53.120e9, "backward_xkb": 101.806e9 + 0.039e9},
-}
+# kernel families (as named in the profile summaries) whose HBM traffic belongs to a class
+FAMILIES = {"forward": ("fwd_lattice", "fwd_mfma"), "backward_xkb": ("bwd_rows_fused", "reduce_columns"),
+            "backward_kb": ("bwdk_rows", "bwdk_mfma"), "backward_x": ("relu_mask", "bwdx_rows")}
+
+
+def profiled_traffic(name):
+    """HBM-side bytes per pass of the network for each kernel class, read from the committed
+    rocprofv3 summary of this workload (profiles/bench_workload_<name>_*.txt, block "HBM-side
+    bytes per pass": FETCH_SIZE + WRITE_SIZE per dispatch, scaled by what the same counters
+    read for a 1 GiB device copy).  Counters cannot be read from inside this script.  Returns
+    ({class: bytes}, file name) or ({}, None) when no summary is there."""
+    import glob
+    import re
+    files = sorted(glob.glob(os.path.join(ROOT, "profiles", f"bench_workload_{name}_*_kernels.txt")))
+    if not files:
+        return {}, None
+    per_family, inside = {}, False
+    with open(files[0]) as fh:
+        for line in fh:
+            if line.startswith("# HBM-side bytes per pass"):
+                inside = True
+                continue
+            if inside:
+                m = re.match(r"#\s+(\S+)\s+([0-9.]+) GB", line)
+                if not m:
+                    break
+                per_family[m.group(1)] = float(m.group(2)) * 1e9
+    out = {}
+    for cls, fams in FAMILIES.items():
+        found = [per_family[f] for f in fams if f in per_family]
+        if found:
+            out[cls] = sum(found)
+    return out, os.path.relpath(files[0], ROOT)
+
 
 WORKLOADS = {
     # name: (kind, ndim, c_in, c_out/labels, depth, width, batch, spatial, adam)
@@ -85,37 +115,46 @@ def make_model(name, torch):
     return model
 
 
-def algorithmic_bytes(name, fused):
-    """Per-step algorithmic bytes of each kernel class, fp32, per layer with C input and
-    w output channels over N voxels:
-    forward (C + w) N 4, backward_x (2C + 2w) N 4, backward_k+bias (C + 2w) N 4, the fused
+def algorithmic_work(name, fused):
+    """Per-step algorithmic bytes and flops of each kernel class, fp32, per layer with C input
+    and w output channels over N voxels and K = 9 or 27 taps:
+    bytes: forward (C + w) N 4, backward_x (2C + 2w) N 4, backward_k+bias (C + 2w) N 4, the fused
     backward_x + backward_k+bias pass (3C + 2w) N 4, each plus the w*C*K weights; the
-    separate ReLU-mask pass of the top layer 3 w N 4 (counted with backward_x).
+    separate ReLU-mask pass of the top layer 3 w N 4 (counted with backward_x);
+    flops: 2 C w K N for each of forward, backward_x and backward_k (the fused pass does two).
     `fused` says which way the library ran the layers above the first (it reports a
-    non-zero call count for the fused class); layer 0 needs no input gradient."""
+    non-zero call count for the fused class); layer 0 needs no input gradient.
+    Returns (bytes per class, flops per class, voxels per step)."""
     kind, ndim, c_in, c_out, depth, width, batch, spatial, adam = WORKLOADS[name]
     n = batch
     for s in spatial:
         n *= s
     K = 3 ** ndim
-    out = {"forward": 0, "backward_x": 3 * width * n * 4, "backward_kb": 0, "backward_xkb": 0}
+    nbytes = {"forward": 0, "backward_x": 3 * width * n * 4, "backward_kb": 0, "backward_xkb": 0}
+    flops = {"forward": 0, "backward_x": 0, "backward_kb": 0, "backward_xkb": 0}
     for i in range(depth):
         C = c_in + width * i
         wts = width * C * K * 4
-        out["forward"] += (C + width) * n * 4 + wts
+        op = 2 * C * width * K * n
+        nbytes["forward"] += (C + width) * n * 4 + wts
+        flops["forward"] += op
         if i > 0 and fused:
-            out["backward_xkb"] += (3 * C + 2 * width) * n * 4 + 2 * wts
+            nbytes["backward_xkb"] += (3 * C + 2 * width) * n * 4 + 2 * wts
+            flops["backward_xkb"] += 2 * op
             continue
         if i > 0:
-            out["backward_x"] += (2 * C + 2 * width) * n * 4 + wts
-        out["backward_kb"] += (C + 2 * width) * n * 4 + wts
-    return out, n
+            nbytes["backward_x"] += (2 * C + 2 * width) * n * 4 + wts
+            flops["backward_x"] += op
+        nbytes["backward_kb"] += (C + 2 * width) * n * 4 + wts
+        flops["backward_kb"] += op
+    return nbytes, flops, n
 
 
 def kernel_times(lib, torch, run_steps):
-    """Per-class kernel time of `run_steps()`: the library brackets every operator
-    launch with HIP events recorded on the launch stream (msd_profile_enable) and
-    msd_profile_read sums the elapsed times after a synchronise."""
+    """Per-class kernel time of `run_steps()`: the library brackets its operator launches
+    with HIP events recorded on the launch stream (msd_profile_enable; inside the block
+    loops one pair of events per run of launches of one class) and msd_profile_read sums the
+    elapsed times after a synchronise."""
     import ctypes
     lib.msd_profile_enable(1)
     run_steps()
@@ -130,13 +169,14 @@ def kernel_times(lib, torch, run_steps):
     return {n: (ms[i], calls[i]) for i, n in enumerate(names)}
 
 
-def cpu_baseline(name, budget_s=15.0):
+def cpu_baseline(name, budget_s=12.0):
     """Time the CPU oracle's dense-block forward+backward on a bounded sample:
     the same network on a smaller image, sized from a calibration run."""
     import torch
     import oracle
     kind, ndim, c_in, c_out, depth, width, batch, spatial, adam = WORKLOADS[name]
-    threads = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
+    host_cpus = os.cpu_count() or 1
+    threads = min(host_cpus, int(os.environ.get("OMP_NUM_THREADS", "16")))
     oracle.set_num_threads(threads)
     torch.manual_seed(0)
     dil = [(i % 10) + 1 for i in range(depth)]
@@ -154,18 +194,110 @@ def cpu_baseline(name, budget_s=15.0):
 
     small = (64, 64) if ndim == 2 else (16, 16, 16)
     t_small = run(small)
-    nv_small = 1
-    for s in small:
-        nv_small *= s
     # scale the edge so the sample costs about budget_s (cost is linear in voxels)
     scale = (budget_s / max(t_small, 1e-6)) ** (1.0 / ndim)
     edge = int(max(small[0], min(small[0] * scale, max(spatial))))
     size = (edge,) * ndim
     t = run(size)
     nv = edge ** ndim
-    return {"value": round(nv / t / 1e6, 4), "unit": "Mvoxel/s", "cores": threads, "kind": "port",
-            "sample": f"C/OpenMP oracle, dense block forward+backward, depth {depth} width {width}, "
-                      f"1x{c_in}x{'x'.join(map(str, size))} fp32, {t:.1f} s"}
+    return {"value": round(nv / t / 1e6, 4), "unit": "Mvoxel/s", "cores": threads, "host_cpus": host_cpus,
+            "kind": "port",
+            "sample": f"C/OpenMP oracle on {threads} threads (the host reports {host_cpus} CPUs), dense block "
+                      f"forward+backward, depth {depth} width {width}, 1x{c_in}x{'x'.join(map(str, size))} "
+                      f"fp32, {t:.1f} s"}
+
+
+def measure(name, args, lib, torch):
+    """One workload: K timed steps, the per-class kernel times of a repeat of them, the
+    roofline of the class that takes the most time, the CPU baseline."""
+    kind, ndim, c_in, c_out, depth, width, batch, spatial, adam = WORKLOADS[name]
+    model = make_model(name, torch)
+    x, target = make_data(name, torch)
+    model.set_input(x)          # inputs resident in HBM before the timed region
+    model.set_target(target)
+
+    # one batch of MSDModel.train: forward, zero_grad, backward and, where the workload has
+    # it, the Adam update, on the batch resident in HBM; like train, the loop does not read
+    # the loss back between steps
+    def step():
+        model.step_async(update=adam)
+
+    eager_step = step
+    if args.graph:
+        from msd_pytorch_amd import GraphedStep
+        if adam:
+            model.optimizer = torch.optim.Adam(model.msd.parameters(), capturable=True)
+        step = GraphedStep(model, update=adam)    # the per-kernel timing below runs the eager step
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+
+    _, _, nvox = algorithmic_work(name, False)
+    result = {
+        "value": round(nvox / (ms_per_step * 1e-3) / 1e6, 3),
+        "unit": "Mvoxel/s",
+        "ms_per_step": round(ms_per_step, 4),
+        "config": {"workload": f"{name}: {DESCRIPTION[name]}", "depth": depth, "width": width,
+                   "batch": batch, "spatial": list(spatial), "hip_graph": bool(args.graph)},
+    }
+
+    if not args.no_kernel_timing:
+        totals = kernel_times(lib, torch, lambda: [eager_step() for _ in range(args.steps)])
+        bytes_per_step, flops_per_step, _ = algorithmic_work(name, totals["backward_xkb"][1] > 0)
+        kernels = {}
+        for cls, (ms, launches) in totals.items():
+            if launches == 0:
+                continue
+            per_step_s = ms / args.steps * 1e-3
+            gbs = bytes_per_step[cls] / per_step_s / 1e9
+            tfl = flops_per_step[cls] / per_step_s / 1e12
+            kernels[cls] = {"ms_per_step": round(per_step_s * 1e3, 4), "calls_per_step": launches // args.steps,
+                            "avg_call_us": round(ms / launches * 1e3, 2),
+                            "algorithmic_GB_per_step": round(bytes_per_step[cls] / 1e9, 3),
+                            "GBps": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4),
+                            "algorithmic_GFLOP_per_step": round(flops_per_step[cls] / 1e9, 2),
+                            "TFLOPs": round(tfl, 2), "frac_fp32": round(tfl / FP32_PEAK_TFLOPS, 4),
+                            "Mvoxel_per_s": round(nvox / per_step_s / 1e6, 2)}
+        dominant = max(kernels, key=lambda c: kernels[c]["ms_per_step"])
+        dom = kernels[dominant]
+        # the committed counter figures describe the library's default launch shapes
+        traffic, source = ({}, None) if args.tune else profiled_traffic(name)
+        per_launch = traffic.get(dominant)
+        by_flops = dom["frac_fp32"] > dom["frac_hbm"]
+        roof = {"bound": "mfma" if by_flops else "hbm", "kernel": dominant,
+                "achieved": dom["TFLOPs"] if by_flops else dom["GBps"],
+                "peak": FP32_PEAK_TFLOPS if by_flops else HBM_PEAK_GBS,
+                "unit": "TFLOP/s" if by_flops else "GB/s",
+                "frac": dom["frac_fp32"] if by_flops else dom["frac_hbm"],
+                # HBM-side bytes per launch (fetch + write counters of the committed rocprofv3
+                # summary), to be compared with the algorithmic bytes per launch
+                "traffic": round(per_launch / dom["calls_per_step"]) if per_launch else None,
+                "traffic_source": source if per_launch else None,
+                "algorithmic_bytes_per_launch": round(bytes_per_step[dominant] / dom["calls_per_step"]),
+                "algorithmic_flops_per_launch": round(flops_per_step[dominant] / dom["calls_per_step"]),
+                "avg_launch_us": dom["avg_call_us"],
+                "hbm": {"achieved_GBps": dom["GBps"], "peak_GBps": HBM_PEAK_GBS, "frac": dom["frac_hbm"]},
+                "fp32": {"achieved_TFLOPs": dom["TFLOPs"], "peak_TFLOPs": FP32_PEAK_TFLOPS, "frac": dom["frac_fp32"],
+                         "pipe": PIPE[dominant]},
+                "timed": "HIP events on the launch stream around the library's operator launches "
+                         "(msd_profile_enable; one pair per run of launches of one class), in a repeat of "
+                         "the K timed steps"}
+        result["roofline"] = roof
+        result["kernels"] = kernels
+        result["hot_path_ms_per_step"] = round(sum(k["ms_per_step"] for k in kernels.values()), 4)
+
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(name)
+    del model
+    torch.cuda.empty_cache()
+    return result
 
 
 def main():
@@ -173,7 +305,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="C", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default=None, choices=sorted(WORKLOADS),
+                    help="one workload only (default: the 2D headline C, then the 3D headline D as 'headline_3d')")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-timing", action="store_true")
     ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
@@ -204,82 +337,20 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    name = args.workload
-    kind, ndim, c_in, c_out, depth, width, batch, spatial, adam = WORKLOADS[name]
-    model = make_model(name, torch)
-    x, target = make_data(name, torch)
-    model.set_input(x)          # inputs resident in HBM before the timed region
-    model.set_target(target)
-
-    # one batch of MSDModel.train: forward, zero_grad, backward and, where the workload has
-    # it, the Adam update, on the batch resident in HBM; like train, the loop does not read
-    # the loss back between steps
-    def step():
-        model.step_async(update=adam)
-
-    eager_step = step
-    if args.graph:
-        from msd_pytorch_amd import GraphedStep
-        if adam:
-            model.optimizer = torch.optim.Adam(model.msd.parameters(), capturable=True)
-        step = GraphedStep(model, update=adam)    # the per-kernel timing below runs the eager step
-
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed / args.steps * 1e3
-
-    _, nvox = algorithmic_bytes(name, False)
+    first = measure(args.workload or "C", args, lib, torch)
     result = {
         "metric": "MSD train-step Mvoxel/s",
-        "value": round(nvox / (ms_per_step * 1e-3) / 1e6, 3),
-        "unit": "Mvoxel/s",
+        "value": first.pop("value"),
+        "unit": first.pop("unit"),
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4),
+        "ms_per_step": first.pop("ms_per_step"),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": f"{name}: {DESCRIPTION[name]}", "depth": depth, "width": width,
-                   "batch": batch, "spatial": list(spatial), "hip_graph": bool(args.graph)},
     }
-
-    if not args.no_kernel_timing:
-        totals = kernel_times(lib, torch, lambda: [eager_step() for _ in range(args.steps)])
-        bytes_per_step, _ = algorithmic_bytes(name, totals["backward_xkb"][1] > 0)
-        kernels = {}
-        for cls, (ms, launches) in totals.items():
-            if launches == 0:
-                continue
-            per_step_ms = ms / args.steps
-            gbs = bytes_per_step[cls] / (per_step_ms * 1e-3) / 1e9
-            kernels[cls] = {"ms_per_step": round(per_step_ms, 4), "calls_per_step": launches // args.steps,
-                            "avg_call_us": round(ms / launches * 1e3, 2),
-                            "algorithmic_GB_per_step": round(bytes_per_step[cls] / 1e9, 3),
-                            "GBps": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4),
-                            "Mvoxel_per_s": round(nvox / (per_step_ms * 1e-3) / 1e6, 2)}
-        dominant = max(kernels, key=lambda c: kernels[c]["ms_per_step"])
-        dom = kernels[dominant]
-        traffic = TRAFFIC.get(name, {}).get(dominant)
-        result["roofline"] = {"bound": "hbm", "kernel": dominant, "achieved": dom["GBps"],
-                              "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom["frac_hbm"],
-                              # HBM-side bytes per launch (fetch + write counters, see TRAFFIC), to be
-                              # compared with the algorithmic bytes per launch that `achieved` is built on
-                              "traffic": round(traffic / dom["calls_per_step"]) if traffic else None,
-                              "algorithmic_bytes_per_launch": round(bytes_per_step[dominant] / dom["calls_per_step"]),
-                              "avg_launch_us": dom["avg_call_us"],
-                              "timed": "HIP events on the launch stream around every operator launch "
-                                       "(msd_profile_enable), in a repeat of the K timed steps"}
-        result["kernels"] = kernels
-        hot = sum(k["ms_per_step"] for k in kernels.values())
-        result["hot_path_ms_per_step"] = round(hot, 4)
-
-    if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(name)
-
+    result.update(first)
+    if args.workload is None:
+        # the metric is quoted on two configurations: the 3D one rides in the same line
+        result["headline_3d"] = measure("D", args, lib, torch)
     print(json.dumps(result))
 
 

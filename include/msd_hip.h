@@ -255,7 +255,9 @@ int msd_block_backward(int dtype, int ndim, int64_t batch, int64_t c_in, int dep
  * block's stack as it is.  weight is contiguous (c_out, c_in), bias (c_out) or NULL.
  * msd_final_backward OVERWRITES grad_input (same layout rules; NULL to skip),
  * grad_weight and grad_bias (either may be NULL); the sums over voxels are reduced in a
- * fixed order through `workspace` (msd_final_workspace_bytes).
+ * fixed order through `workspace` (msd_final_workspace_bytes); with grad_weight and
+ * grad_bias both NULL (a frozen layer) the input is not read (it may be NULL) and no
+ * workspace is needed.
  */
 int64_t msd_final_workspace_bytes(int dtype, int64_t batch, int64_t c_in, int64_t c_out, int64_t nvox);
 int msd_final_forward(int dtype, int64_t batch, int64_t c_in, int64_t c_out, int64_t nvox,
@@ -271,8 +273,10 @@ int msd_final_backward(int dtype, int64_t batch, int64_t c_in, int64_t c_out, in
                        void *workspace, int64_t workspace_bytes, void *stream);
 
 /*
- * Kernel timing for benchmarks.  While enabled, every operator call (also inside
- * the block calls) is bracketed by HIP events recorded on its launch stream.
+ * Kernel timing for benchmarks.  While enabled, every operator call is bracketed by
+ * HIP events recorded on its launch stream; inside the block calls consecutive launches
+ * of one class share one pair of events (a pair per launch would add its own few
+ * microseconds of idle stream to every launch).
  * msd_profile_read waits for the recorded events and returns, per class
  * {0 forward, 1 backward_x incl. the mask, 2 backward_k/bias, 3 fused backward_x +
  * backward_k/bias of the block backward pass}, the summed elapsed milliseconds and the

@@ -38,8 +38,8 @@ template <typename T> struct is_f32 { static constexpr bool value = false; };
 template <> struct is_f32<float> { static constexpr bool value = true; };
 
 // Optional per-class kernel timing with HIP events recorded on the launch stream
-// (msd_profile_* in the C ABI).  Classes: 0 forward, 1 backward_x (+ mask), 2 backward_k/bias.
-constexpr int kProfileClasses = 4;   // forward, backward_x, backward_k(+bias), fused backward_x+k
+// (msd_profile_* in the C ABI).
+constexpr int kProfileClasses = 4;   // forward, backward_x (+ mask), backward_k(+bias), fused backward_x+k
 
 struct Profile {
     bool on = false;
@@ -47,17 +47,35 @@ struct Profile {
     size_t used = 0;
     struct Span {
         size_t start, stop;                                  // indices into pool
-        bool counted;                                        // adds to the class's number of calls
+        int64_t calls;                                       // operator calls the span covers
     };
     std::vector<Span> spans[kProfileClasses];
-    hipEvent_t take()
+    // Inside a block loop (ProfileBatch) consecutive launches of one class share ONE pair of
+    // events, and the event that ends a run starts the next one: a pair per launch costs about
+    // four microseconds of idle stream per launch, which would be charged to the kernels.
+    bool batching = false;
+    int open_cls = -1;
+    size_t open_start = 0;
+    int64_t open_calls = 0;
+
+    // index of a fresh event recorded on s, or SIZE_MAX
+    size_t record(hipStream_t s)
     {
         if (used == pool.size()) {
             hipEvent_t e;
-            if (hipEventCreate(&e) != hipSuccess) return nullptr;
+            if (hipEventCreate(&e) != hipSuccess) return SIZE_MAX;
             pool.push_back(e);
         }
-        return pool[used++];
+        if (hipEventRecord(pool[used], s) != hipSuccess) return SIZE_MAX;
+        return used++;
+    }
+    // ends the open run of a batch (if any) at a new event and returns that event's index
+    size_t close_run(hipStream_t s)
+    {
+        const size_t e = record(s);
+        if (open_cls >= 0 && e != SIZE_MAX) spans[open_cls].push_back({open_start, e, open_calls});
+        open_cls = -1;
+        return e;
     }
 } g_profile;
 
@@ -68,21 +86,50 @@ struct ProfileScope {
     int cls;
     hipStream_t s;
     size_t start = 0;
-    bool active, counted;
-    ProfileScope(int cls_, hipStream_t s_, bool counted_ = true)
-        : cls(cls_), s(s_), active(g_profile.on), counted(counted_)
+    bool active;
+    int64_t calls;
+    ProfileScope(int cls_, hipStream_t s_, bool counted = true)
+        : cls(cls_), s(s_), active(g_profile.on), calls(counted ? 1 : 0)
     {
         if (!active) return;
-        start = g_profile.used;
-        hipEvent_t e = g_profile.take();
-        if (!e || hipEventRecord(e, s) != hipSuccess) active = false;
+        if (g_profile.batching) {
+            active = false;                       // the run's events do the timing
+            if (g_profile.open_cls != cls) {
+                const size_t e = g_profile.close_run(s);
+                if (e == SIZE_MAX) return;
+                g_profile.open_cls = cls;
+                g_profile.open_start = e;
+                g_profile.open_calls = 0;
+            }
+            g_profile.open_calls += calls;
+            return;
+        }
+        start = g_profile.record(s);
+        if (start == SIZE_MAX) active = false;
     }
     ~ProfileScope()
     {
         if (!active) return;
-        const size_t stop = g_profile.used;
-        hipEvent_t e = g_profile.take();
-        if (e && hipEventRecord(e, s) == hipSuccess) g_profile.spans[cls].push_back({start, stop, counted});
+        const size_t stop = g_profile.record(s);
+        if (stop != SIZE_MAX) g_profile.spans[cls].push_back({start, stop, calls});
+    }
+};
+
+// For the lifetime of this object the scopes on stream s are merged into runs per class.
+struct ProfileBatch {
+    hipStream_t s;
+    bool active;
+    explicit ProfileBatch(hipStream_t s_) : s(s_), active(g_profile.on && !g_profile.batching)
+    {
+        if (!active) return;
+        g_profile.batching = true;
+        g_profile.open_cls = -1;
+    }
+    ~ProfileBatch()
+    {
+        if (!active) return;
+        if (g_profile.open_cls >= 0) g_profile.close_run(s);
+        g_profile.batching = false;
     }
 };
 
@@ -721,6 +768,7 @@ int msd_block_forward(int dtype, int ndim, int64_t batch, int64_t c_in, int dept
     MSD_TRY(check_block(fn, dtype, ndim, batch, c_in, depth, widths, spatial, dilations, stack, stack_strides,
                         weights, &a));
     if (!bias) return fail(MSD_ERR_INVALID, "%s: bias is NULL", fn);
+    ProfileBatch profile_runs((hipStream_t)stream);
     int64_t first = c_in, b0 = 0;
     for (int i = 0; i < depth; i++) {
         char *out = (char *)stack + first * stack_strides[1] * a.elem;
@@ -749,6 +797,7 @@ int msd_block_backward(int dtype, int ndim, int64_t batch, int64_t c_in, int dep
                         weights, &a));
     if (!grads || !grads_strides || !grad_weights) return fail(MSD_ERR_INVALID, "%s: NULL argument", fn);
     int64_t last = a.c_total, b1 = a.c_total - c_in;
+    ProfileBatch profile_runs((hipStream_t)stream);
     DeferredReductions pending;
     pending.s = (hipStream_t)stream;
     const int64_t layer_ws = block_layer_workspace(dtype, ndim, batch, c_in, depth, widths, spatial);
@@ -856,12 +905,15 @@ int msd_final_backward(int dtype, int64_t batch, int64_t c_in, int64_t c_out, in
 {
     const char *fn = "final_backward";
     MSD_TRY(check_final(fn, dtype, batch, c_in, c_out, nvox));
-    if (!input || !weight || !grad_output) return fail(MSD_ERR_INVALID, "%s: NULL argument", fn);
+    if (!weight || !grad_output) return fail(MSD_ERR_INVALID, "%s: NULL argument", fn);
+    if (!input && (grad_weight || grad_bias))
+        return fail(MSD_ERR_INVALID, "%s: input is NULL (it may only be omitted when grad_input is the only gradient)", fn);
     if (input_batch_stride < 0 || input_channel_stride < 0 || grad_output_batch_stride < 0 ||
         grad_output_channel_stride < 0 || grad_input_batch_stride < 0 || grad_input_channel_stride < 0)
         return fail(MSD_ERR_INVALID, "%s: negative stride", fn);
-    const int64_t need = msd_final_workspace_bytes(dtype, batch, c_in, c_out, nvox);
-    if (!workspace || workspace_bytes < need)
+    // the workspace holds the partial sums of the weight and bias gradients: not needed for grad_input alone
+    const int64_t need = grad_weight || grad_bias ? msd_final_workspace_bytes(dtype, batch, c_in, c_out, nvox) : 0;
+    if (need > 0 && (!workspace || workspace_bytes < need))
         return fail(MSD_ERR_WORKSPACE, "%s: workspace of %lld bytes needed, %lld given", fn, (long long)need,
                     (long long)(workspace ? workspace_bytes : 0));
     const hipError_t e =
@@ -883,6 +935,8 @@ int msd_final_backward(int dtype, int64_t batch, int64_t c_in, int64_t c_out, in
 int msd_profile_enable(int on)
 {
     g_profile.on = on != 0;
+    g_profile.batching = false;
+    g_profile.open_cls = -1;
     g_profile.used = 0;
     for (auto &v : g_profile.spans) v.clear();
     return MSD_OK;
@@ -900,7 +954,7 @@ int msd_profile_read(double *ms, int64_t *calls)
             if (e == hipSuccess) e = hipEventElapsedTime(&t, g_profile.pool[sp.start], g_profile.pool[sp.stop]);
             if (e != hipSuccess) return hip_fail("msd_profile_read", e);
             total += t;
-            ncalls += sp.counted ? 1 : 0;
+            ncalls += sp.calls;
         }
         ms[c] = total;
         calls[c] = ncalls;

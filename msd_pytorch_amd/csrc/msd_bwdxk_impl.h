@@ -500,6 +500,8 @@ size_t lds_bytes(const RowTeams &rt, const RowSegments &sg)
     return std::max(main_loop, epilogue);
 }
 
+constexpr size_t kMaxLdsBytes = 64 * 1024;
+
 // Strides and in-plane offsets fit the kernel's 32-bit arithmetic.
 template <typename T>
 inline bool small_strides(const Geom &g, const View<T> &v)
@@ -519,8 +521,16 @@ bool fits(const Geom &g, int V, const View<const float> &gy, const View<const fl
     RowSegments sg;
     // the plain kernel loads x in aligned groups of four voxels; the LONG one from any address
     if (lng ? g.W < 4 : (g.W % 4 != 0 || !rows_aligned(x, g.W, 4))) return false;
+    sg = RowSegments{1, 0};
     if (!make_row_teams(g, V, &rt, lng ? &sg : nullptr)) return false;
     if (rt.lpr % kWave != 0 || rt.lpr * rt.rpw > kThreads) return false;
+    // staged rows + the waves' A tiles within the 64 KB of LDS a workgroup may ask for without
+    // opting in to more (3D rows of 512 voxels at two voxels per lane would take 77 KB: such
+    // rows are cut into segments by the LONG instances instead)
+    const size_t kr = (size_t)g.Wd * Taps<NDIM>::K + 1;
+    const size_t main_loop = ((size_t)rt.rpw * g.Wd * RowTaps<NDIM>::NPQ * (V * rt.lpr + sg.halo) +
+                              (size_t)kWaves * kr * (kWave * V + 4)) * 4;
+    if (main_loop > kMaxLdsBytes) return false;
     return rows_aligned(gy, g.W, V) && rows_aligned(gx, g.W, V);
 }
 
@@ -573,6 +583,7 @@ hipError_t launch(const Geom &g, const View<const float> &gy, const View<const f
     a.want_bias = gb != nullptr;
     const int chunks = (g.C + NCB * kChanBlock - 1) / (NCB * kChanBlock);
     const size_t lds = lds_bytes<NDIM, V, NCB, WOUT>(a.rt, a.sg);
+    if (lds > kMaxLdsBytes) return hipErrorInvalidConfiguration;   // excluded by fits()
     hipLaunchKernelGGL((bwd_rows_fused<NDIM, V, NCB, WOUT, LONG>), dim3(rows, 1, chunks), dim3(a.rt.lpr * a.rt.rpw), lds, s, a,
                        gy.p, x.p, gx.p, actp, k, part);
     hipError_t e = hipGetLastError();

@@ -117,21 +117,26 @@ __global__ __launch_bounds__(kFinalThreads) void final_backward_kernel(int64_t n
 #pragma unroll
         for (int e = 0; e < V; e++) g[o][e] = keep ? g[o][e] : T(0);
     }
+    // part == nullptr: neither the weight nor the bias gradient is wanted (a frozen layer);
+    // the input is then not read at all and only grad_input is written
+    const bool want_sums = part != nullptr;       // uniform
     // bias gradient: sum of the output gradient over voxels
+    if (want_sums) {
 #pragma unroll
-    for (int o = 0; o < MAXO; o++) {
-        T s = T(0);
+        for (int o = 0; o < MAXO; o++) {
+            T s = T(0);
 #pragma unroll
-        for (int e = 0; e < V; e++) s += g[o][e];
-        s = wave_sum(s);
-        if (lane == 0 && o0 + o < c_out) part[((int64_t)c_out * C + o0 + o) * rows + row] = s;
+            for (int e = 0; e < V; e++) s += g[o][e];
+            s = wave_sum(s);
+            if (lane == 0 && o0 + o < c_out) part[((int64_t)c_out * C + o0 + o) * rows + row] = s;
+        }
     }
     const T *xp = x + (int64_t)b * xsb + ic * V;
     T *gp = gx ? gx + (int64_t)b * gxsb + ic * V : nullptr;
 #pragma unroll 2
     for (int c = 0; c < C; c++) {
         T v[V];
-        load_elems<T, V>(xp + (int64_t)c * xsc, v);
+        if (want_sums) load_elems<T, V>(xp + (int64_t)c * xsc, v);
         if (gp) {
             T r[V];
             if (o0 > 0) {                         // later groups of output channels add to the first one's result
@@ -148,13 +153,15 @@ __global__ __launch_bounds__(kFinalThreads) void final_backward_kernel(int64_t n
             }
             if (active) store_elems<T, V>(gp + (int64_t)c * gxsc, r);
         }
+        if (want_sums) {
 #pragma unroll
-        for (int o = 0; o < MAXO; o++) {
-            T s = T(0);
+            for (int o = 0; o < MAXO; o++) {
+                T s = T(0);
 #pragma unroll
-            for (int e = 0; e < V; e++) s += g[o][e] * v[e];
-            s = wave_sum(s);
-            if (lane == 0 && o0 + o < c_out) part[((int64_t)(o0 + o) * C + c) * rows + row] = s;
+                for (int e = 0; e < V; e++) s += g[o][e] * v[e];
+                s = wave_sum(s);
+                if (lane == 0 && o0 + o < c_out) part[((int64_t)(o0 + o) * C + c) * rows + row] = s;
+            }
         }
     }
 }
@@ -251,6 +258,8 @@ hipError_t final_backward(int64_t batch, int c_in, int c_out, int64_t nvox, cons
     const int64_t nvec = nvox / V;
     const dim3 grid((unsigned)((nvec + kFinalThreads - 1) / kFinalThreads), (unsigned)batch, 1);
     const int64_t rows = (int64_t)grid.x * batch * (kFinalThreads / kWave);
+    if (!gw && !gb) ws = nullptr;                 // no sums over voxels wanted: no partial sums, no second pass
+    if (!ws && !gx) return hipSuccess;
     for (int o0 = 0; o0 < c_out;) {
         const int gwd = group_width(c_out - o0);
 #define MSD_FINAL_BWD(VV, OO)                                                                                        \
@@ -267,6 +276,7 @@ hipError_t final_backward(int64_t batch, int c_in, int c_out, int64_t nvox, cons
         if (e != hipSuccess) return e;
         o0 += gwd;
     }
+    if (!ws) return hipSuccess;
     const int64_t nw = (int64_t)c_out * c_in, ncols = nw + c_out;
     hipLaunchKernelGGL(final_reduce_kernel<T>, dim3((unsigned)ncols), dim3(256), 0, s, ws, rows, nw, ncols, gw, gb);
     return hipGetLastError();

@@ -10,6 +10,7 @@ The tensors' device pointers, sizes and strides are handed to the C ABI of
 chosen by the library for gfx950.
 """
 import ctypes
+import operator
 
 import torch
 
@@ -74,13 +75,20 @@ def _check_dim(fn, name, t, dim):
 
 
 def _check_dilation(fn, t, dilation):
-    """checkDilation (msd_custom_convolutions.cpp:39-52)."""
-    if not isinstance(dilation, int) or isinstance(dilation, bool):
+    """checkDilation (msd_custom_convolutions.cpp:39-52).  Returns the dilation as a Python
+    int: like the reference's pybind11 int caster, any integer type is accepted (numpy and
+    torch integer scalars), bool and float are not."""
+    if isinstance(dilation, (bool, float)):
         raise TypeError(f"{fn}: dilation must be an int")
+    try:
+        dilation = operator.index(dilation)
+    except TypeError:
+        raise TypeError(f"{fn}: dilation must be an int") from None
     if dilation <= 0:
         _fail(fn, "Dilation must be 1 or greater")
     if any(dilation > s for s in t.shape[2:]):
         _fail(fn, "Dilation cannot be greater than size of image. ")
+    return dilation
 
 
 def _check_block_size(fn, block_size):
@@ -136,7 +144,7 @@ def _forward(fn, native, input, kernel, bias, output, dilation, block_size):
         _fail(fn, "Kernel shape does not match output channels. ")
     if bias.shape[0] != output.shape[1]:
         _fail(fn, "Bias shape does not match output channels. ")
-    _check_dilation(fn, input, dilation)
+    dilation = _check_dilation(fn, input, dilation)
     _check_block_size(fn, block_size)
     bias = bias.contiguous()
     _call(native, input.device, *_head(input, input.shape[1], output.shape[1], dilation), *_view(input),
@@ -171,7 +179,7 @@ def _backward_x(fn, native, output, grad_output, kernel, grad_input, dilation, b
         _fail(fn, "Kernel shape does not match input channels. ")
     if kernel.shape[0] != grad_output.shape[1] or (relu and kernel.shape[0] != output.shape[1]):
         _fail(fn, "Kernel shape does not match output channels. ")
-    _check_dilation(fn, grad_input, dilation)
+    dilation = _check_dilation(fn, grad_input, dilation)
     _check_block_size(fn, block_size)
     head = _head(grad_input, grad_input.shape[1], grad_output.shape[1], dilation)
     views = (*_view(output),) if relu else ()
@@ -218,7 +226,7 @@ def _backward_k(fn, native, output, grad_output, input, grad_kernel, grad_bias, 
             _fail(fn, "Bias shape does not match output channels. ")
         if not grad_bias.is_contiguous():
             _fail(fn, "Expected grad_bias to be contiguous")
-    _check_dilation(fn, input, dilation)
+    dilation = _check_dilation(fn, input, dilation)
     _check_block_size(fn, block_size)
     c_in, c_out = input.shape[1], grad_output.shape[1]
     ws, ws_ptr, ws_bytes = _workspace(input, c_in, c_out)
@@ -282,7 +290,7 @@ def conv_backward_xkb(grad_output, input, kernel, grad_input, grad_kernel, grad_
     if grad_bias is not None and (grad_bias.dim() != 1 or grad_bias.shape[0] != grad_output.shape[1]
                                   or not grad_bias.is_contiguous()):
         _fail(fn, "Bias shape does not match output channels. ")
-    _check_dilation(fn, input, dilation)
+    dilation = _check_dilation(fn, input, dilation)
     _check_block_size(fn, block_size)
     c_in, c_out = input.shape[1], grad_output.shape[1]
     ws, ws_ptr, ws_bytes = _workspace(input, c_in, c_out)
@@ -359,18 +367,20 @@ def _check_block(fn, stack, c_in, dilations, bias, weights):
     if len(dilations) != len(weights):
         _fail(fn, "number of weights does not match depth")
     channels = c_in
+    checked = []
     for i, (w, d) in enumerate(zip(weights, dilations)):
         _check_kernel(fn, w)
         _check_dim(fn, f"weight{i}", w, stack.dim())
         if w.shape[1] != channels:
             _fail(fn, "Kernel shape does not match input channels. ")
-        _check_dilation(fn, stack, d)
+        checked.append(_check_dilation(fn, stack, d))
         channels += w.shape[0]
     if channels != stack.shape[1]:
         _fail(fn, "Kernel shape does not match output channels. ")
     _check_dim(fn, "bias", bias, 1)
     if bias.shape[0] != channels - c_in:
         _fail(fn, "Bias shape does not match output channels. ")
+    return checked
 
 
 def _block_head(stack, c_in, dilations, weights):
@@ -388,7 +398,7 @@ def block_forward(stack, c_in, dilations, bias, weights):
     hold the block's input.  Layer i: conv_relu_forward(stack[:, :C_i], weights[i],
     bias slice, stack[:, C_i:C_i + width_i], dilations[i])."""
     fn = "block_forward"
-    _check_block(fn, stack, c_in, dilations, bias, weights)
+    dilations = _check_block(fn, stack, c_in, dilations, bias, weights)
     bias = bias.contiguous()
     _call("msd_block_forward", stack.device, *_block_head(stack, c_in, dilations, weights), *_view(stack),
           _ptr_array(weights), ctypes.c_void_p(bias.data_ptr()), _stream(stack))
@@ -400,9 +410,9 @@ def block_backward(stack, grads, c_in, dilations, weights, grad_weights, grad_bi
     dL/dinput.  ``grad_weights[i]`` (zero-filled, or None to skip) and ``grad_bias``
     (zero-filled, or None) are accumulated into."""
     fn = "block_backward"
-    _check_block(fn, stack, c_in, dilations, torch.empty(stack.shape[1] - c_in, dtype=stack.dtype,
-                                                          device=stack.device) if grad_bias is None else grad_bias,
-                 weights)
+    dilations = _check_block(fn, stack, c_in, dilations,
+                             torch.empty(stack.shape[1] - c_in, dtype=stack.dtype, device=stack.device)
+                             if grad_bias is None else grad_bias, weights)
     named = [("stack", stack), ("grads", grads)] + [(f"grad_weight{i}", g) for i, g in enumerate(grad_weights)
                                                     if g is not None]
     _check_same_gpu(fn, named)
@@ -472,11 +482,15 @@ def final_forward(input, weight, bias, output):
 
 def final_backward(input, grad_output, weight, grad_input, grad_weight, grad_bias):
     """Gradients of final_forward; grad_input (or None), grad_weight (or None) and
-    grad_bias (or None) are OVERWRITTEN."""
+    grad_bias (or None) are OVERWRITTEN.  ``input`` may be None when neither grad_weight nor
+    grad_bias is wanted (a frozen layer): grad_input does not depend on it."""
     fn = "final_backward"
-    named = [("input", input), ("grad_output", grad_output), ("weight", weight)]
-    named += [(n, t) for n, t in (("grad_input", grad_input), ("grad_weight", grad_weight), ("grad_bias", grad_bias))
-              if t is not None]
+    if input is None and (grad_weight is not None or grad_bias is not None or grad_input is None):
+        _fail(fn, "input may only be omitted when grad_input is the only gradient wanted")
+    shaped = input if input is not None else grad_input
+    named = [("grad_output", grad_output), ("weight", weight)]
+    named += [(n, t) for n, t in (("input", input), ("grad_input", grad_input), ("grad_weight", grad_weight),
+                                  ("grad_bias", grad_bias)) if t is not None]
     _check_same_gpu(fn, named)
     _check_same_type(fn, named)
     c_out, c_in = weight.shape[0], weight.shape[1]
@@ -486,26 +500,29 @@ def final_backward(input, grad_output, weight, grad_input, grad_weight, grad_bia
         _fail(fn, "Expected grad_weight to be contiguous and shaped like weight")
     if grad_bias is not None and (grad_bias.numel() != c_out or not grad_bias.is_contiguous()):
         _fail(fn, "Expected grad_bias to be contiguous with c_out elements")
-    if input.shape[1] != c_in or grad_output.shape[1] != c_out or input.shape[0] != grad_output.shape[0] \
-            or tuple(input.shape[2:]) != tuple(grad_output.shape[2:]):
+    if shaped.shape[1] != c_in or grad_output.shape[1] != c_out or shaped.shape[0] != grad_output.shape[0] \
+            or tuple(shaped.shape[2:]) != tuple(grad_output.shape[2:]):
         _fail(fn, "Input shape does not match output shape. ")
-    if grad_input is not None and tuple(grad_input.shape) != tuple(input.shape):
+    if grad_input is not None and tuple(grad_input.shape) != tuple(shaped.shape):
         _fail(fn, "Input shape does not match output shape. ")
     for t in (input, grad_output, grad_input):
         if t is not None and not final_layer_supported(t):
             _fail(fn, "Expected channel planes to be contiguous")
-    nvox, isb, isc = _flat_strides(input)
+    nvox, isb, isc = _flat_strides(shaped)
     _, gsb, gsc = _flat_strides(grad_output)
     xsb, xsc = (grad_input.stride(0), grad_input.stride(1)) if grad_input is not None else (0, 0)
-    lib = _native.load()
-    need = lib.msd_final_workspace_bytes(_DTYPES[input.dtype], input.shape[0], c_in, c_out, nvox)
-    if need < 0:
-        _fail(fn, _native.last_error())
-    ws = torch.empty(max(int(need), 8), dtype=torch.uint8, device=input.device)
+    need, ws = 0, None
+    if grad_weight is not None or grad_bias is not None:
+        # partial sums of the weight and bias gradients (fixed-order reduction)
+        need = _native.load().msd_final_workspace_bytes(_DTYPES[shaped.dtype], shaped.shape[0], c_in, c_out, nvox)
+        if need < 0:
+            _fail(fn, _native.last_error())
+        ws = torch.empty(max(int(need), 8), dtype=torch.uint8, device=shaped.device)
 
     def ptr(t):
         return ctypes.c_void_p(t.data_ptr() if t is not None else 0)
 
+    input = shaped      # only its geometry is used when the caller passed None
     _call("msd_final_backward", input.device, _DTYPES[input.dtype], input.shape[0], c_in, c_out, nvox, ptr(input), isb,
           isc, ptr(grad_output), gsb, gsc, ptr(weight), ptr(grad_input), xsb, xsc, ptr(grad_weight), ptr(grad_bias),
           ptr(ws), int(need), _stream(input))

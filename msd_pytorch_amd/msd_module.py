@@ -29,7 +29,10 @@ class MSDFinalFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, input, weight, bias):
-        ctx.save_for_backward(input, weight)
+        # the input is only needed for the weight and bias gradients: a frozen layer (the
+        # models' scaling layers) does not keep the activation alive
+        ctx.save_for_backward(input if any(ctx.needs_input_grad[1:]) else None, weight)
+        ctx.input_shape = input.shape
         output = torch.empty(input.shape[0], weight.shape[0], *input.shape[2:], dtype=input.dtype,
                              device=input.device)
         cc.final_forward(input, weight, bias, output)
@@ -40,7 +43,8 @@ class MSDFinalFunction(torch.autograd.Function):
         input, weight = ctx.saved_tensors
         if not cc.final_layer_supported(grad_output):
             grad_output = grad_output.contiguous()
-        grad_input = torch.empty_like(input) if ctx.needs_input_grad[0] else None
+        grad_input = torch.empty(ctx.input_shape, dtype=weight.dtype, device=weight.device) \
+            if ctx.needs_input_grad[0] else None
         grad_weight = torch.empty_like(weight) if ctx.needs_input_grad[1] else None
         grad_bias = torch.empty(weight.shape[0], dtype=weight.dtype, device=weight.device) \
             if ctx.needs_input_grad[2] else None

@@ -1,0 +1,95 @@
+"""Parity checks shared by the GPU test files: one operator problem, or one dense block,
+run through the HIP library (C ABI) and through the CPU oracle on the same seeded data.
+
+Tolerances (max |diff| / max |ref|, fp32): forward 1e-5, gradients 1e-4."""
+import torch
+
+import oracle
+from cases import make_problem, rel_err
+
+
+def bias_close(got, want, terms, tol=1e-4):
+    """A bias gradient is one long sum per channel, which may cancel to almost nothing: the
+    error is measured against a hundredth of the sum of the magnitudes at least."""
+    floor = 0.01 * terms.abs().double().sum(dim=[0] + list(range(2, terms.dim()))).max().item()
+    diff = (got.double().cpu() - want.double()).abs().max().item()
+    return diff <= tol * max(want.abs().max().item(), floor)
+
+
+def check_operator_problem(cc, shape, seed=7):
+    """conv_relu_forward, the three conv_relu_backward_* operators (accumulating) and the
+    three plain backward operators as one call (conv_backward_xkb), against the oracle."""
+    ref = make_problem(shape, torch.float32, seed=seed)
+    dev = make_problem(shape, torch.float32, device="cuda", seed=seed)
+    d = ref["d"]
+    oracle.conv_relu_forward(ref["x"], ref["k"], ref["bias"], ref["y"], d)
+    cc.conv_relu_forward(dev["x"], dev["k"], dev["bias"], dev["y"], d)
+    assert rel_err(dev["stack"], ref["stack"]) <= 1e-5, "conv_relu_forward"
+    assert torch.equal(dev["x"].cpu(), ref["x"]), "conv_relu_forward wrote outside its output channels"
+    dev["y"].copy_(ref["y"])                    # same mask on both sides
+    want_gk, want_gb = torch.ones_like(ref["k"]), torch.full_like(ref["bias"], -1.0)
+    oracle.conv_relu_backward_x(ref["y"], ref["gy"], ref["k"], ref["gx"], d)
+    oracle.conv_relu_backward_k(ref["y"], ref["gy"], ref["x"], want_gk, d)
+    oracle.conv_relu_backward_bias(ref["y"], ref["gy"], want_gb)
+    got_gk, got_gb = torch.ones_like(dev["k"]), torch.full_like(dev["bias"], -1.0)
+    cc.conv_relu_backward_x(dev["y"], dev["gy"], dev["k"], dev["gx"], d)
+    cc.conv_relu_backward_k(dev["y"], dev["gy"], dev["x"], got_gk, d)
+    cc.conv_relu_backward_bias(dev["y"], dev["gy"], got_gb)
+    torch.cuda.synchronize()
+    assert rel_err(dev["gstack"], ref["gstack"]) <= 1e-4, "conv_relu_backward_x"
+    assert torch.equal(dev["gy"].cpu(), ref["gy"]), "conv_relu_backward_x wrote outside grad_input"
+    assert rel_err(got_gk, want_gk) <= 1e-4, "conv_relu_backward_k"
+    assert bias_close(got_gb, want_gb, ref["gy"] * (ref["y"] > 0)), "conv_relu_backward_bias"
+    # the three plain operators in one call
+    ref2 = make_problem(shape, torch.float32, seed=seed + 1)
+    dev2 = make_problem(shape, torch.float32, device="cuda", seed=seed + 1)
+    want_gk, want_gb = torch.zeros_like(ref2["k"]), torch.zeros_like(ref2["bias"])
+    oracle.conv_backward_x(ref2["gy"], ref2["k"], ref2["gx"], d)
+    oracle.conv_backward_k(ref2["gy"], ref2["x"], want_gk, d)
+    oracle.conv_backward_bias(ref2["gy"], want_gb)
+    got_gk, got_gb = torch.zeros_like(dev2["k"]), torch.zeros_like(dev2["bias"])
+    cc.conv_backward_xkb(dev2["gy"], dev2["x"], dev2["k"], dev2["gx"], got_gk, got_gb, d)
+    torch.cuda.synchronize()
+    assert rel_err(dev2["gstack"], ref2["gstack"]) <= 1e-4, "conv_backward_xkb grad_input"
+    assert rel_err(got_gk, want_gk) <= 1e-4, "conv_backward_xkb grad_kernel"
+    assert bias_close(got_gb, want_gb, ref2["gy"]), "conv_backward_xkb grad_bias"
+
+
+def block_problem(ndim, size, c_in, width, depth, batch, dilations=None, seed=0):
+    """Input, dilations (1..10 in turn unless given), bias, weights and the gradient of the
+    whole stack, fp32 on the CPU."""
+    gen = torch.Generator().manual_seed(seed)
+    dil = list(dilations) if dilations is not None else [min((i % 10) + 1, min(size)) for i in range(depth)]
+    taps = 3 ** ndim
+    ws = [torch.randn(width, c_in + width * i, *([3] * ndim), generator=gen)
+          * (2.0 / (taps * (c_in + width * max(depth - 1, 1)) + 1)) ** 0.5 for i in range(depth)]
+    bias = torch.randn(width * depth, generator=gen) * 0.05
+    x = torch.rand(batch, c_in, *size, generator=gen)
+    g = torch.randn(batch, c_in + width * depth, *size, generator=gen)
+    return x, dil, bias, ws, g
+
+
+def check_block(ndim, size, c_in, width, depth, batch, dilations=None, seed=0):
+    """msd_block forward + backward (native layer loops) against the fp64 oracle: the whole
+    stack, grad_input, every weight gradient and the bias gradient."""
+    from msd_pytorch_amd.msd_block import msd_block
+    x, dil, bias, ws, g = block_problem(ndim, size, c_in, width, depth, batch, dilations, seed)
+    xd = x.cuda().requires_grad_(True)
+    bd = bias.cuda().requires_grad_(True)
+    wd = [w.cuda().requires_grad_(True) for w in ws]
+    got = msd_block(xd, dil, bd, *wd)
+    got.backward(g.cuda())
+    torch.cuda.synchronize()
+    ws64 = [w.double() for w in ws]
+    want = oracle.block_forward(x.double(), dil, bias.double(), ws64)
+    assert rel_err(got, want) <= 1e-5, "stack"
+    del want
+    # The backward oracle takes its ReLU masks from the stack the GPU computed: an activation
+    # within rounding of zero may have the other sign in double precision, and one flipped
+    # mask in an upper layer changes every gradient below it by far more than the tolerance.
+    want_gx, want_gb, want_gw = oracle.block_backward(got.detach().double().cpu(), g.double(), dil, bias.double(),
+                                                      ws64)
+    assert rel_err(xd.grad, want_gx) <= 1e-4, "grad_input"
+    assert rel_err(bd.grad, want_gb) <= 1e-4, "grad_bias"
+    worst = max((rel_err(a.grad, b), i) for i, (a, b) in enumerate(zip(wd, want_gw)))
+    assert worst[0] <= 1e-4, "grad_weight of layer %d" % worst[1]

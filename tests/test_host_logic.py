@@ -85,6 +85,19 @@ def test_cpu_tensors_are_rejected_like_the_reference():
         cc.conv_relu_backward_kb(x, x, x, torch.zeros(1, 1, 3, 3), torch.zeros(1), 1)
 
 
+def test_dilation_accepts_any_integer_type():
+    # the reference's pybind11 int caster takes numpy and torch integer scalars
+    # (MSDModule(dilations=np.arange(1, 11)) works upstream); bool and float are refused
+    import numpy as np
+    img = torch.zeros(1, 1, 8, 8)
+    for d in (3, np.int64(3), np.int32(3), torch.tensor(3), np.arange(1, 11)[2]):
+        got = cc._check_dilation("f", img, d)
+        assert got == 3 and type(got) is int
+    for bad in (True, 2.0, np.float32(2), "2", None):
+        with pytest.raises(TypeError):
+            cc._check_dilation("f", img, bad)
+
+
 def test_check_helpers_raise_runtime_error():
     with pytest.raises(RuntimeError, match="Dilation must be 1 or greater"):
         cc._check_dilation("f", torch.zeros(1, 1, 4, 4), 0)

@@ -1,0 +1,94 @@
+"""Every launch-shape setting of msd_set_tuning against the CPU oracle.
+
+The library picks voxels per lane, rows per forward tile, channel groups, tile numbering and
+workgroup order by image size; each choice is a different template instance or code path, and
+some are reached by default only at particular sizes.  Here every setting is forced in turn on
+problems small enough for the oracle, so that each instance meets the oracle at least once
+whatever the defaults are.  Results may only differ in floating-point summation order:
+tolerances forward 1e-5, gradients 1e-4 (fp32)."""
+import itertools
+
+import pytest
+import torch
+
+from parity import check_block, check_operator_problem
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def cc():
+    from msd_pytorch_amd import msd_custom_convolutions
+    return msd_custom_convolutions
+
+
+class tuning:
+    """Sets the given knobs for the duration of a with-block, then restores the defaults."""
+
+    def __init__(self, settings):
+        from msd_pytorch_amd import _native
+        self.lib = _native.load()
+        self.settings = settings
+
+    def __enter__(self):
+        for key, value in self.settings.items():
+            assert self.lib.msd_set_tuning(key.encode(), value) == 0, key
+        return self
+
+    def __exit__(self, *exc):
+        for key in self.settings:
+            self.lib.msd_set_tuning(key.encode(), -1)
+        return False
+
+
+# (B, C_in, C_out, spatial, dilation)
+IMG_A = (1, 5, 1, (23, 256), 3)          # rows of 256: 64 lanes at 4 voxels per lane
+IMG_B = (2, 18, 1, (9, 1024), 7)         # one row per workgroup, two blocks of 16 channels, folds in y
+IMG_C = (1, 35, 2, (12, 512), 5)         # two output channels, three channel blocks
+IMG_D = (1, 3, 1, (70, 128), 1)          # dilation 1, many row groups
+VOL_A = (1, 6, 1, (7, 9, 128), 2)
+VOL_B = (1, 19, 1, (5, 6, 256), 3)       # rows of 256: up to 4 voxels per lane in the forward pass
+VOL_C = (2, 4, 2, (6, 7, 128), 1)        # two output channels
+VOL_D = (1, 3, 1, (40, 40, 64), 1)       # more than 128 lattices per residue class: tiles in 4 x 4 blocks
+VOL_E = (1, 17, 1, (24, 20, 64), 3)      # lattices of 3 x 3 rows
+
+FORWARD_2D = [({"fwd.rows2d": r, "fwd.vec2d": v}, s)
+              for r, v in itertools.product((2, 3, 4, 5, 6), (1, 2, 4)) for s in (IMG_A, IMG_B)]
+FORWARD_2D += [({"fwd.vec2d": v}, IMG_C) for v in (1, 2, 4)]
+FORWARD_3D = [({"fwd.vec3d": v}, s) for v in (1, 2, 4) for s in (VOL_A, VOL_B, VOL_C)]
+FORWARD_3D += [({"fwd.class3d": c}, s) for c in (0, 1) for s in (VOL_A, VOL_D, VOL_E)]
+SPLIT = [({"fwd.split": k}, s) for k in (1, 2, 4) for s in (IMG_A, IMG_C, VOL_A, VOL_C)]
+ORDER = [({"xcd_remap": r}, s) for r in (0, 1) for s in (IMG_B, IMG_D, VOL_A, VOL_D)]
+BACKWARD_K = [({"bwdk.vec2d": v}, s) for v in (1, 2, 4) for s in (IMG_A, IMG_B, IMG_C)]
+BACKWARD_K += [({"bwdk.vec3d": v}, s) for v in (1, 2) for s in (VOL_A, VOL_B)]
+BACKWARD_K += [({"bwdk.rows": r}, s) for r in (0, 1) for s in (IMG_A, IMG_B, VOL_A)]
+BACKWARD_K += [({"bwdk.rows": 0, "bwdk.vec2d": v}, IMG_B) for v in (2, 4)]
+BACKWARD_K += [({"bwdk.interleave": i}, s) for i in (0, 1) for s in (IMG_D, VOL_D)]
+BACKWARD_K += [({"bwdk.blocks": n}, s) for n in (8, 40) for s in (IMG_D, VOL_A)]
+BACKWARD_X = [({"bwdx.vec2d": v, "bwdx.unroll2d": u}, s) for v in (1, 2, 4) for u in (2, 4) for s in (IMG_A, IMG_C)]
+BACKWARD_X += [({"bwdx.vec3d": v, "bwdx.unroll3d": u}, s) for v in (1, 2, 4) for u in (2, 4) for s in (VOL_B, VOL_C)]
+BACKWARD_X += [({"bwdx.min_blocks": n}, s) for n in (1, 4096) for s in (IMG_B, VOL_B)]
+
+
+def _id(case):
+    settings, s = case
+    knobs = ",".join("%s=%d" % kv for kv in settings.items())
+    return "%s-B%d-C%d-w%d-%s-d%d" % (knobs, s[0], s[1], s[2], "x".join(map(str, s[3])), s[4])
+
+
+@pytest.mark.parametrize("case", FORWARD_2D + FORWARD_3D + SPLIT + ORDER + BACKWARD_K + BACKWARD_X, ids=_id)
+def test_operators_under_a_forced_setting(cc, case):
+    settings, shape = case
+    with tuning(settings):
+        check_operator_problem(cc, shape, seed=3)
+
+
+BLOCK_SETTINGS = [{"block.snake": 0}, {"block.snake": 1}, {"block.fuse": 0}, {"block.defer": 0},
+                  {"xcd_remap": 0}, {"bwdk.interleave": 0}, {"fwd.class3d": 0}]
+
+
+@pytest.mark.parametrize("settings", BLOCK_SETTINGS, ids=lambda s: ",".join("%s=%d" % kv for kv in s.items()))
+@pytest.mark.parametrize("ndim,size", [(2, (21, 256)), (3, (6, 9, 128))])
+def test_block_under_a_forced_setting(ndim, size, settings):
+    with tuning(settings):
+        check_block(ndim, size, 2, 1, 19, 2)

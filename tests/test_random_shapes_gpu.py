@@ -8,7 +8,8 @@ import pytest
 import torch
 
 import oracle
-from cases import make_problem, rel_err
+from cases import rel_err
+from parity import check_operator_problem
 
 pytestmark = pytest.mark.gpu
 
@@ -82,46 +83,7 @@ def _extreme_cases(seed, n):
     s[0], s[1], s[2], "x".join(map(str, s[3])), s[4]))
 def test_random_operator_problems(shape):
     from msd_pytorch_amd import msd_custom_convolutions as cc
-    ref = make_problem(shape, torch.float32, seed=7)
-    dev = make_problem(shape, torch.float32, device="cuda", seed=7)
-    d = ref["d"]
-    # forward with ReLU, then the three ReLU backward operators (accumulating)
-    oracle.conv_relu_forward(ref["x"], ref["k"], ref["bias"], ref["y"], d)
-    cc.conv_relu_forward(dev["x"], dev["k"], dev["bias"], dev["y"], d)
-    assert rel_err(dev["stack"], ref["stack"]) <= 1e-5, "conv_relu_forward"
-    dev["y"].copy_(ref["y"])                    # same mask on both sides
-    want_gk, want_gb = torch.ones_like(ref["k"]), torch.full_like(ref["bias"], -1.0)
-    oracle.conv_relu_backward_x(ref["y"], ref["gy"], ref["k"], ref["gx"], d)
-    oracle.conv_relu_backward_k(ref["y"], ref["gy"], ref["x"], want_gk, d)
-    oracle.conv_relu_backward_bias(ref["y"], ref["gy"], want_gb)
-    got_gk, got_gb = torch.ones_like(dev["k"]), torch.full_like(dev["bias"], -1.0)
-    cc.conv_relu_backward_x(dev["y"], dev["gy"], dev["k"], dev["gx"], d)
-    cc.conv_relu_backward_k(dev["y"], dev["gy"], dev["x"], got_gk, d)
-    cc.conv_relu_backward_bias(dev["y"], dev["gy"], got_gb)
-    torch.cuda.synchronize()
-    assert rel_err(dev["gstack"], ref["gstack"]) <= 1e-4, "conv_relu_backward_x"
-    assert rel_err(got_gk, want_gk) <= 1e-4, "conv_relu_backward_k"
-    # a bias gradient is one long sum per channel, which may cancel to almost nothing: the
-    # error is then measured against a hundredth of the sum of the magnitudes at least
-    terms = (ref["gy"] * (ref["y"] > 0)).abs().double().sum(dim=[0] + list(range(2, ref["gy"].dim())))
-    floor = 0.01 * terms.max().item()
-    diff = (got_gb.double().cpu() - want_gb.double()).abs().max().item()
-    assert diff <= 1e-4 * max(want_gb.abs().max().item(), floor), "conv_relu_backward_bias"
-    # the three plain operators in one call
-    ref2 = make_problem(shape, torch.float32, seed=8)
-    dev2 = make_problem(shape, torch.float32, device="cuda", seed=8)
-    want_gk, want_gb = torch.zeros_like(ref2["k"]), torch.zeros_like(ref2["bias"])
-    oracle.conv_backward_x(ref2["gy"], ref2["k"], ref2["gx"], d)
-    oracle.conv_backward_k(ref2["gy"], ref2["x"], want_gk, d)
-    oracle.conv_backward_bias(ref2["gy"], want_gb)
-    got_gk, got_gb = torch.zeros_like(dev2["k"]), torch.zeros_like(dev2["bias"])
-    cc.conv_backward_xkb(dev2["gy"], dev2["x"], dev2["k"], dev2["gx"], got_gk, got_gb, d)
-    torch.cuda.synchronize()
-    assert rel_err(dev2["gstack"], ref2["gstack"]) <= 1e-4, "conv_backward_xkb grad_input"
-    assert rel_err(got_gk, want_gk) <= 1e-4, "conv_backward_xkb grad_kernel"
-    floor = 0.01 * ref2["gy"].abs().double().sum(dim=[0] + list(range(2, ref2["gy"].dim()))).max().item()
-    diff = (got_gb.double().cpu() - want_gb.double()).abs().max().item()
-    assert diff <= 1e-4 * max(want_gb.abs().max().item(), floor), "conv_backward_xkb grad_bias"
+    check_operator_problem(cc, shape)
 
 
 def _block_cases(seed, n):
