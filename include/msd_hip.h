@@ -175,6 +175,25 @@ int msd_conv_relu_backward_kb(int dtype, int ndim, int64_t batch, int64_t c_in, 
                               void *grad_kernel, void *grad_bias,
                               void *workspace, int64_t workspace_bytes, void *stream);
 
+/* msd_conv_relu_backward_kb without a workspace argument and without any allocation.
+ * No counterpart in the reference.  It is for callers that cannot allocate device memory:
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * The partial sums of the fixed-order reduction go through a buffer of
+ * MSD_STATIC_SCRATCH_BYTES = 32 MiB that is part of the library's device image (each GPU
+ * the library runs on holds it until the process ends); a problem whose msd_workspace_bytes
+ * exceeds it is rejected with MSD_ERR_WORKSPACE and nothing is launched.  Same kernels and
+ * the same bits as msd_conv_relu_backward_kb.  All calls on one GPU share the buffer: calls
+ * that overlap on one GPU (different streams or threads) race.  The first call on a device
+ * looks the buffer's address up (hipGetSymbolAddress) and so must not be made under stream
+ * capture; later calls only launch kernels. */
+#define MSD_STATIC_SCRATCH_BYTES (32 * 1024 * 1024)
+int msd_conv_relu_backward_kb_static(int dtype, int ndim, int64_t batch, int64_t c_in, int64_t c_out,
+                                     const int64_t *spatial, int dilation,
+                                     const void *output, const int64_t *output_strides,
+                                     const void *grad_output, const int64_t *grad_output_strides,
+                                     const void *input, const int64_t *input_strides,
+                                     void *grad_kernel, void *grad_bias, void *stream);
+
 /* msd_conv_backward_k and msd_conv_backward_bias in one pass (no ReLU mask).
  * grad_bias may be NULL.  No counterpart in the reference. */
 int msd_conv_backward_kb(int dtype, int ndim, int64_t batch, int64_t c_in, int64_t c_out,

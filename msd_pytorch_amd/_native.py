@@ -11,6 +11,7 @@ ABI_VERSION = 1
 
 MSD_F32, MSD_F64 = 0, 1
 MSD_OK, MSD_ERR_INVALID, MSD_ERR_HIP, MSD_ERR_WORKSPACE = 0, 1, 2, 3
+STATIC_SCRATCH_BYTES = 32 * 1024 * 1024   # MSD_STATIC_SCRATCH_BYTES of the header
 
 _c_int = ctypes.c_int
 _c_i64 = ctypes.c_int64
@@ -38,6 +39,7 @@ PROTOTYPES = {
     "msd_conv_relu_backward_bias": (_c_int, [_c_int, _c_int, _c_i64, _c_i64, _i64p] + _VIEW + _VIEW + [_ptr]
                                     + _WS + [_ptr]),
     "msd_conv_relu_backward_kb": (_c_int, _HEAD + _VIEW + _VIEW + _VIEW + [_ptr, _ptr] + _WS + [_ptr]),
+    "msd_conv_relu_backward_kb_static": (_c_int, _HEAD + _VIEW + _VIEW + _VIEW + [_ptr, _ptr, _ptr]),
     "msd_conv_backward_kb": (_c_int, _HEAD + _VIEW + _VIEW + [_ptr, _ptr] + _WS + [_ptr]),
     "msd_conv_backward_xkb": (_c_int, _HEAD + _VIEW + _VIEW + [_ptr] + _VIEW + [_ptr, _ptr] + _WS + [_ptr]),
     "msd_relu_mask_gradient": (_c_int, [_c_int, _c_int, _c_i64, _c_i64, _i64p] + _VIEW + _VIEW + [_ptr]),

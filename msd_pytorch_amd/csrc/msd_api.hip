@@ -6,6 +6,7 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <mutex>
 #include <string>
 #include <utility>
 #include <vector>
@@ -594,6 +595,69 @@ int msd_conv_relu_backward_kb(int dtype, int ndim, int64_t batch, int64_t c_in, 
                        workspace, workspace_bytes, stream);
 }
 
+
+// ---------------------------------------------------------------------------
+// msd_conv_relu_backward_kb for callers that cannot allocate: the partial sums go through
+// a buffer that is part of the library's device image instead of a caller's workspace.
+// ---------------------------------------------------------------------------
+
+// One copy per GPU the library runs on, held until the process ends.  In host code this name
+// is only a handle for hipGetSymbolAddress: it is not a device address.
+static __device__ __align__(256) __attribute__((used)) unsigned char scratch[MSD_STATIC_SCRATCH_BYTES];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices];   // device address of `scratch` on device i, once looked up
+
+// Address of the current device's copy of `scratch` (looked up on the first call on each
+// device, with that device current).
+int static_scratch(const char *fn, void **ptr)
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_fail(fn, e);
+    if (dev < 0 || dev >= kMaxDevices) return fail(MSD_ERR_INVALID, "%s: device index %d not supported", fn, dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return hip_fail(fn, e);
+        if (!p) return fail(MSD_ERR_HIP, "%s: the static scratch buffer has no device address", fn);
+        g_scratch_ptr[dev] = p;
+    }
+    *ptr = g_scratch_ptr[dev];
+    return MSD_OK;
+}
+
+}  // namespace
+
+int msd_conv_relu_backward_kb_static(int dtype, int ndim, int64_t batch, int64_t c_in, int64_t c_out,
+                                     const int64_t *spatial, int dilation, const void *output,
+                                     const int64_t *output_strides, const void *grad_output,
+                                     const int64_t *grad_output_strides, const void *input,
+                                     const int64_t *input_strides, void *grad_kernel, void *grad_bias, void *stream)
+{
+    const char *fn = "conv_relu_backward_kb_static";
+    // geometry and size first: these rejections touch no device
+    msd::Geom g;
+    MSD_TRY(make_geom(fn, dtype, ndim, batch, c_in, c_out, spatial, dilation, true, &g));
+    if (c_in <= 0) return fail(MSD_ERR_INVALID, "%s: c_in must be positive", fn);
+    const int64_t need = msd::generic_workspace_elems(g) * (dtype == MSD_F32 ? 4 : 8);
+    if (need > MSD_STATIC_SCRATCH_BYTES)
+        return fail(MSD_ERR_WORKSPACE,
+                    "%s: this problem needs %lld bytes of scratch, the library's static buffer holds %lld; "
+                    "call msd_conv_relu_backward_kb with a workspace instead",
+                    fn, (long long)need, (long long)MSD_STATIC_SCRATCH_BYTES);
+    void *ws = nullptr;
+    MSD_TRY(static_scratch(fn, &ws));
+    // the kernels write every partial sum (and every value of the masked gradient) that the
+    // second pass reads, so nothing in the buffer has to start at zero
+    return backward_kb(fn, true, true, dtype, ndim, batch, c_in, c_out, spatial, dilation, output, output_strides,
+                       grad_output, grad_output_strides, input, input_strides, grad_kernel, grad_bias, ws,
+                       MSD_STATIC_SCRATCH_BYTES, stream);
+}
 
 // ---------------------------------------------------------------------------
 // Dense block: the layer loops of msd_block.py:40-58 (forward) and :89-130

@@ -229,12 +229,16 @@ def _backward_k(fn, native, output, grad_output, input, grad_kernel, grad_bias, 
     dilation = _check_dilation(fn, input, dilation)
     _check_block_size(fn, block_size)
     c_in, c_out = input.shape[1], grad_output.shape[1]
-    ws, ws_ptr, ws_bytes = _workspace(input, c_in, c_out)
     head = _head(input, c_in, c_out, dilation)
     views = (*_view(output),) if relu else ()
     grads = (ctypes.c_void_p(grad_kernel.data_ptr()),)
-    if native in ("msd_conv_relu_backward_kb", "msd_conv_backward_kb"):
+    if native in ("msd_conv_relu_backward_kb", "msd_conv_backward_kb", "msd_conv_relu_backward_kb_static"):
         grads += (ctypes.c_void_p(grad_bias.data_ptr() if grad_bias is not None else 0),)
+    if native == "msd_conv_relu_backward_kb_static":
+        # the library's own scratch buffer: nothing is allocated for this call
+        _call(native, input.device, *head, *views, *_view(grad_output), *_view(input), *grads, _stream(input))
+        return
+    ws, ws_ptr, ws_bytes = _workspace(input, c_in, c_out)
     _call(native, input.device, *head, *views, *_view(grad_output), *_view(input), *grads, ws_ptr, ws_bytes,
           _stream(input))
 
@@ -256,6 +260,15 @@ def conv_relu_backward_kb(output, grad_output, input, grad_kernel, grad_bias, di
     calls msd_block.py:113-126 makes per layer).  Not part of the reference's module."""
     _backward_k("conv_relu_backward_kb", "msd_conv_relu_backward_kb", output, grad_output, input, grad_kernel,
                 grad_bias, dilation, block_size)
+
+
+def conv_relu_backward_kb_static(output, grad_output, input, grad_kernel, grad_bias, dilation, block_size=None):
+    """conv_relu_backward_kb for callers that cannot allocate device memory (HIP graph
+    capture, serving loops): the partial sums go through a 32 MiB buffer inside the library
+    instead of a workspace tensor.  Raises RuntimeError for problems that need more; calls
+    that overlap on one GPU race.  Not part of the reference's module."""
+    _backward_k("conv_relu_backward_kb_static", "msd_conv_relu_backward_kb_static", output, grad_output, input,
+                grad_kernel, grad_bias, dilation, block_size)
 
 
 def conv_backward_kb(grad_output, input, grad_kernel, grad_bias, dilation, block_size=None):

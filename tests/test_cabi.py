@@ -82,6 +82,23 @@ def test_backward_k_rejects_missing_workspace():
     assert "workspace" in _native.last_error()
 
 
+def test_static_scratch_entry_point_rejects_before_touching_the_device():
+    # msd_conv_relu_backward_kb_static: geometry errors and problems larger than the
+    # library's scratch buffer are refused before any HIP call
+    lib = _native.load()
+    s2, s3 = i64(1, 1, 1, 1), i64(1, 1, 1, 1, 1)
+    null = ctypes.c_void_p(0)
+    rc = lib.msd_conv_relu_backward_kb_static(0, 2, 1, 1, 1, i64(4, 4), 5, FAKE, s2, FAKE, s2, FAKE, s2, FAKE, null, null)
+    assert rc == _native.MSD_ERR_INVALID and "Dilation cannot be greater" in _native.last_error()
+    big = i64(256, 256, 256)
+    assert lib.msd_workspace_bytes(0, 3, 1, 2, 1, big) > _native.STATIC_SCRATCH_BYTES
+    rc = lib.msd_conv_relu_backward_kb_static(0, 3, 1, 2, 1, big, 1, FAKE, s3, FAKE, s3, FAKE, s3, FAKE, null, null)
+    assert rc == _native.MSD_ERR_WORKSPACE and "static buffer" in _native.last_error()
+    header = open(HEADER).read()
+    assert "#define MSD_STATIC_SCRATCH_BYTES (32 * 1024 * 1024)" in header
+    assert _native.STATIC_SCRATCH_BYTES == 32 * 1024 * 1024
+
+
 def test_workspace_query():
     lib = _native.load()
     n32 = lib.msd_workspace_bytes(0, 2, 1, 10, 1, i64(64, 64))
