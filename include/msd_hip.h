@@ -76,7 +76,8 @@ int msd_set_kernel_path(int path);
  * workgroups take every n-th row group), "block.fuse" (0/1: fused backward in the block),
  * "block.defer" (0/1: one reduction launch for many layers), "block.snake" (0/1: alternate
  * layers walk the channels in opposite directions), "fwd.class3d" (0/1: 3D forward tiles
- * numbered by residue class).  Unknown keys return MSD_ERR_INVALID.
+ * numbered by residue class), "fwd.lattice3d" (24, 33 or 44: rows z x y of a 3D forward tile;
+ * 0: chosen by the library).  Unknown keys return MSD_ERR_INVALID.
  */
 int msd_set_tuning(const char *key, int value);
 

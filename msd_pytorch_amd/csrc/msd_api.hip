@@ -16,9 +16,9 @@ const char *const kKnobNames[kKnobCount] = {
     "bwdx.vec2d", "bwdx.vec3d", "bwdx.unroll2d", "bwdx.unroll3d", "bwdx.min_blocks",
     "xcd_remap", "bwdk.vec2d", "bwdk.vec3d", "bwdk.blocks",
     "fwd.vec2d", "fwd.vec3d", "fwd.split", "fwd.rows2d", "bwdk.rows", "block.fuse",
-    "block.defer", "bwdk.interleave", "block.snake", "fwd.class3d",
+    "block.defer", "bwdk.interleave", "block.snake", "fwd.class3d", "fwd.lattice3d",
 };
-static_assert(kKnobFwdClass3d + 1 == kKnobCount, "one name per knob, in the order of the enum");
+static_assert(kKnobFwdLattice3d + 1 == kKnobCount, "one name per knob, in the order of the enum");
 int g_knobs[kKnobCount];
 // every knob starts at "library default"
 const bool g_knobs_ready = [] {

@@ -34,6 +34,13 @@
 
 #include <type_traits>
 
+#ifndef MSD_XPAIR
+#define MSD_XPAIR 1
+#endif
+#ifndef MSD_PIPELINE_SETS_EXPR
+#define MSD_PIPELINE_SETS_EXPR 2
+#endif
+
 namespace msd {
 namespace bwdxk {
 
@@ -78,6 +85,17 @@ template <int NDIM, int V, int NCB, int WOUT> constexpr int resident_per_cu()
     return (NDIM == 3 && V == 1 && WOUT == 1 && NCB <= 4) ? 3 : 2;
 }
 
+// Register sets of the channel loop's load pipeline: the loads of stage s + NSETS - 1 are
+// issued before the arithmetic of stage s.  A stage is short (a few hundred cycles of
+// arithmetic on 2 to 4 KB per wave), so with one stage of lead a wave has at most two stages
+// in flight, which at the memory latency under load is not enough to fill the memory
+// system; a set costs 8 (3D) to 16 (2D, four voxels per lane) registers.  Four sets where
+// they fit without costing a resident workgroup.
+template <int NDIM, int V, int NCB, int WOUT, bool LONG> constexpr int pipeline_sets()
+{
+    return MSD_PIPELINE_SETS_EXPR;
+}
+
 // LONG: the variant for what the plain kernel's 32-bit lane offsets and whole-row teams do
 // not reach.  The first channel of each block of 16 moves into the uniform base of the x
 // loads (so the stack may be of any size and its rows need not be aligned or whole groups of four
@@ -102,6 +120,16 @@ void bwd_rows_fused(const Args a, const float *__restrict__ gyp, const float *__
     constexpr int NSS = V == 1 ? (NCB <= 4 ? 1 : 2) : (V == 4 ? 2 : 4);
     constexpr int H = 4 * V / NSS;                // stages per block of 16 channels (even)
     constexpr int NCS = kChanBlock / H;           // grad_input channels per stage
+    constexpr int NSETS = pipeline_sets<NDIM, V, NCB, WOUT, LONG>();   // register sets of the load pipeline
+    // 16-voxel stages (one voxel per lane): the x loads of a stage take 64 bytes per channel, half
+    // a cache line, and by the time the next stage asks for the other half the line has left the
+    // 32 KB vector cache again, so every line of x crosses from the L2 twice; the vector cache's
+    // outstanding misses are what bounds the kernel.  XPAIR: x is requested for two stages at a
+    // time (both halves of a line together), the rest of the stage (grad_input channels,
+    // arithmetic) stays at 16 voxels.
+    constexpr bool XPAIR = NDIM == 3 && V == 1 && NSS == 1 && !LONG && MSD_XPAIR;
+    static_assert(!XPAIR || (H == 4 && NSETS == 2), "a block is two pairs of stages");
+    static_assert(H % NSETS == 0 && NSETS >= 2, "the stages of a block rotate through the register sets");
     constexpr int ASTRIDE = ATile<NDIM, V, WOUT>::kStride;
     const Geom &g = a.g;
     const RowTeams &rt = a.rt;
@@ -187,8 +215,8 @@ void bwd_rows_fused(const Args a, const float *__restrict__ gyp, const float *__
         // ---- one pipeline stage of loads: NSS 16-voxel groups of 16 channels of x in the MFMA B
         // layout, and NCS channels of grad_input in the voxel layout.  Clamped, always valid
         // addresses; what does not count is replaced after the load.
-        float ka[NSS][4], kb[NSS][4];             // stages alternate between the a and b buffers
-        float ga[NCS][V], gb[NCS][V];
+        float xs_[NSETS][NSS][4];                 // stage s uses set s % NSETS
+        float gs_[NSETS][NCS][V];
         auto load_stage = [&](int cb, int h, float (&kk)[NSS][4], float (&gg)[NCS][V]) {
             // (redefining the lane offset keeps its widening to 64 bits next to the loads, where
             // it is free; hoisted out of the loop it would make every address a vector addition)
@@ -213,9 +241,33 @@ void bwd_rows_fused(const Args a, const float *__restrict__ gyp, const float *__
                 load_global_vec<V>(channel_base(gbase, ci), goff, gg[j]);
             }
         };
+        // XPAIR: x of the pair of 16-voxel groups 2 * pair, 2 * pair + 1 (one cache line per channel) ...
+        auto load_x2 = [&](int cb, int pair, float (&kk)[2][4]) {
+            const uint32_t xch = (uint32_t)min(c0 + cb * kChanBlock + mj, g.C - 1) * (uint32_t)xsc + xrow;
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+                load_global_vec<4>(xbase, 4u * (xch + (uint32_t)min(kx + 16 * (2 * pair + j), g.W - 4)), kk[j]);
+        };
+        // ... and the grad_input channels of stage h
+        auto load_g = [&](int cb, int h, float (&gg)[NCS][V]) {
+            asm volatile("" : "+v"(goff));
+#pragma unroll
+            for (int j = 0; j < NCS; j++) {
+                const int ci = max(min(c0 + cb * kChanBlock + h * NCS + j, cx_end - 1), 0);
+                load_global_vec<V>(channel_base(gbase, ci), goff, gg[j]);
+            }
+        };
+        float xpa[2][4], xpb[2][4];               // XPAIR: the two pairs of a block alternate
         // block of 16 channels that stage `s` of the walk belongs to
         auto block_of = [&](int s) { return g.reverse ? ncb - 1 - s / H : s / H; };
-        load_stage(block_of(0), 0, ka, ga);   // issued ahead of the gather so the two latencies overlap
+        // issued ahead of the gather so the latencies overlap (a tile has at least H >= NSETS stages)
+        if constexpr (XPAIR) {
+            load_x2(block_of(0), 0, xpa);
+            load_g(block_of(0), 0, gs_[0]);
+        } else {
+#pragma unroll
+            for (int q = 0; q < NSETS - 1; q++) load_stage(block_of(q), q % H, xs_[q], gs_[q]);
+        }
 
         // ---- A operands, voxel layout: tv[co * K + t][i] = A_co[t](voxel x0 + i of the team's row)
         float tv[KR][V];
@@ -375,33 +427,77 @@ void bwd_rows_fused(const Args a, const float *__restrict__ gyp, const float *__
             }
         };
 
-        // ---- channel loop: blocks of 16 channels, H stages each, two stages per iteration; the
-        // loads of the next stage are issued before the arithmetic of the current one
-        const int nst = ncb * H;                  // even
+        // ---- channel loop: blocks of 16 channels, H stages each, NSETS stages per iteration (all of
+        // one block); the loads of stage s + NSETS - 1 are issued before the arithmetic of stage s
+        const int nst = ncb * H;                  // a multiple of NSETS
+        if constexpr (XPAIR) {
+            // one block of 16 channels (four stages) per iteration.  Every load is issued a stage
+            // or more ahead of its use and none sits behind a test (loads retire in order, and the
+            // compiler sizes each wait for the path with the fewest loads behind the one it needs):
+            // past the last block the loads ask for lines of this block again.
 #pragma unroll 1
-        for (int st = 0; st < nst; st += 2) {
-            const int cb = block_of(st), h = st % H;
-            load_stage(cb, h + 1, kb, gb);
+            for (int blk = 0; blk < ncb; blk++) {
+                const int cb = g.reverse ? ncb - 1 - blk : blk;
+                const bool more = blk + 1 < ncb;
+                const int cbn = more ? (g.reverse ? cb - 1 : cb + 1) : cb;
+#pragma unroll
+                for (int tg = 0; tg < TG; tg++)
+#pragma unroll
+                    for (int c = 0; c < NCH; c++) acc[tg][c] = mfma4{0.f, 0.f, 0.f, 0.f};
+                load_g(cb, 1, gs_[1]);
+                load_x2(cb, 1, xpb);
+                stage_k(cb, 0, reinterpret_cast<float (&)[NSS][4]>(xpa[0]));
+                stage_x(cb, 0, gs_[0]);
+                load_g(cb, 2, gs_[0]);
+                stage_k(cb, 1, reinterpret_cast<float (&)[NSS][4]>(xpa[1]));
+                stage_x(cb, 1, gs_[1]);
+                load_g(cb, 3, gs_[1]);
+                load_x2(cbn, more ? 0 : 1, xpa);
+                stage_k(cb, 2, reinterpret_cast<float (&)[NSS][4]>(xpb[0]));
+                stage_x(cb, 2, gs_[0]);
+                load_g(cbn, more ? 0 : 3, gs_[0]);
+                stage_k(cb, 3, reinterpret_cast<float (&)[NSS][4]>(xpb[1]));
+                stage_x(cb, 3, gs_[1]);
+#pragma unroll
+                for (int q = 0; q < NCB; q++)
+                    if (q == cb) {
+#pragma unroll
+                        for (int tg = 0; tg < TG; tg++)
+#pragma unroll
+                            for (int c = 0; c < NCH; c++) D[q][tg] += acc[tg][c];
+                    }
+            }
+        } else
+#pragma unroll 1
+        for (int st = 0; st < nst; st += NSETS) {
+            const int cb = block_of(st);
 #pragma unroll
             for (int tg = 0; tg < TG; tg++)
 #pragma unroll
                 for (int c = 0; c < NCH; c++) acc[tg][c] = mfma4{0.f, 0.f, 0.f, 0.f};
-            stage_k(cb, h, ka);
-            stage_x(cb, h, ga);
-            // 2D: no test around these loads.  Loads and stores retire through one in-order
-            // counter and the compiler derives each wait from what may be pending on any path,
-            // so a load that may be skipped turns the wait in front of the next matrix
-            // instructions into one for these loads themselves.  The last iteration loads its
-            // own first stage again instead (cache hits, never used).  Measured: 2 % faster in
-            // 2D, 2 % slower in 3D (fewer, longer iterations per tile), which keeps the test.
-            if constexpr (NDIM == 2) {
-                const int sn = min(st + 2, nst - 2);
-                load_stage(block_of(sn), sn % H, ka, ga);
-            } else {
-                if (st + 2 < nst) load_stage(block_of(st + 2), (st + 2) % H, ka, ga);
+#pragma unroll
+            for (int u = 0; u < NSETS; u++) {
+                const int h = st % H + u;
+                constexpr int kLead = NSETS - 1;
+                float (&kn)[NSS][4] = xs_[(u + kLead) % NSETS];
+                float (&gn)[NCS][V] = gs_[(u + kLead) % NSETS];
+                // 2D: no test around these loads.  Loads and stores retire through one in-order
+                // counter and the compiler derives each wait from what may be pending on any path,
+                // so a load that may be skipped turns the wait in front of the next matrix
+                // instructions into one for these loads themselves.  Past the last stage a stage
+                // of this tile is loaded again instead (cache hits, never used).  Measured with two
+                // sets: 2 % faster in 2D, 2 % slower in 3D (fewer, longer iterations per tile),
+                // which keeps the test.
+                if constexpr (NDIM == 2) {
+                    const int sn = min(st + u + kLead, nst - 1);
+                    load_stage(block_of(sn), sn % H, kn, gn);
+                } else {
+                    const int sn = st + u + kLead;
+                    if (sn < nst) load_stage(block_of(sn), sn % H, kn, gn);
+                }
+                stage_k(cb, h, xs_[u]);
+                stage_x(cb, h, gs_[u]);
             }
-            stage_k(cb, h + 1, kb);
-            stage_x(cb, h + 1, gb);
             // D is indexed statically: pick the block with a chain of uniform branches
 #pragma unroll
             for (int q = 0; q < NCB; q++)

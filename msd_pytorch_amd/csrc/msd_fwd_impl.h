@@ -41,20 +41,13 @@ struct Lattice {
     int by_class;   // 3D: tiles numbered residue class by residue class (2: a class row by row, no blocks)
 };
 
-template <int NDIM, bool RELU, int WOUT, int V, int RZ, int RY>
-__global__ __launch_bounds__(NDIM == 3 ? 512 : 1024, (NDIM == 3 && V == 1 && WOUT == 1) ? 8 : 1) void fwd_lattice(Geom g, Lattice lt, int remap, View<const float> x,
-                                                    const float *__restrict__ k, const float *__restrict__ bias,
-                                                    View<float> out)
+// First output row (y0, z0) of the lattice this workgroup computes; false for the padding
+// blocks of the grid and for lattices that start past the image (uniform over the workgroup).
+template <int NDIM, int RZ, int RY>
+__device__ __forceinline__ bool tile_origin(const Geom &g, const Lattice &lt, int remap, int &y0, int &z0)
 {
-    extern __shared__ float lds[];
-    constexpr int K = Taps<NDIM>::K;
-    constexpr int NZ = Taps<NDIM>::NZ;          // z taps: 3 or 1
-    constexpr int LZ = NDIM == 3 ? RZ + 2 : 1;  // input lattice levels along z
-    constexpr int LY = RY + 2;
-    static_assert(NDIM == 3 || RZ == 1, "2D has a single z level");
-
     const int tile = block_for_xcd(blockIdx.x, gridDim.x, remap);
-    if (tile >= lt.ntiles) return;               // padding block
+    if (tile >= lt.ntiles) return false;         // padding block
     // 3D: tiles are numbered in blocks of kOrder x kOrder (y, z) neighbours.  Neighbouring
     // lattices share a third of their input rows, and only tiles that start together walk the
     // channels in step and find each other's rows in the L2.
@@ -77,7 +70,7 @@ __global__ __launch_bounds__(NDIM == 3 ? 512 : 1024, (NDIM == 3 && V == 1 && WOU
         const int cls = tile / per_class, rem = tile % per_class;
         const int blk = rem / (kOrder * kOrder), within = rem % (kOrder * kOrder);
         const int sy = (blk % bys) * kOrder + within % kOrder, sz = (blk / bys) * kOrder + within / kOrder;
-        if (sy >= lt.segs_y || sz >= lt.segs_z) return;     // padding of the block grid (whole workgroup)
+        if (sy >= lt.segs_y || sz >= lt.segs_z) return false;   // padding of the block grid
         ty = (cls % g.dil) * lt.segs_y + sy;
         tz = (cls / g.dil) * lt.segs_z + sz;
     } else if (NDIM == 3) {
@@ -85,14 +78,30 @@ __global__ __launch_bounds__(NDIM == 3 ? 512 : 1024, (NDIM == 3 && V == 1 && WOU
         const int nby = (lt.tiles_y + kOrder - 1) / kOrder;
         ty = (blk % nby) * kOrder + within % kOrder;
         tz = (blk / nby) * kOrder + within / kOrder;
-        if (ty >= lt.tiles_y || tz >= lt.tiles_z) return;   // padding of the block grid (whole workgroup)
+        if (ty >= lt.tiles_y || tz >= lt.tiles_z) return false;   // padding of the block grid
     } else {
         ty = tile;
         tz = 0;
     }
-    const int y0 = ty / lt.segs_y + (ty % lt.segs_y) * RY * g.dil;
-    const int z0 = NDIM == 3 ? tz / lt.segs_z + (tz % lt.segs_z) * RZ * g.dil : 0;
-    if (y0 >= g.H || z0 >= g.D) return;          // empty tail of a residue class (whole workgroup)
+    y0 = ty / lt.segs_y + (ty % lt.segs_y) * RY * g.dil;
+    z0 = NDIM == 3 ? tz / lt.segs_z + (tz % lt.segs_z) * RZ * g.dil : 0;
+    return y0 < g.H && z0 < g.D;                 // false: empty tail of a residue class
+}
+
+template <int NDIM, bool RELU, int WOUT, int V, int RZ, int RY>
+__global__ __launch_bounds__(NDIM == 3 ? 512 : 1024, (NDIM == 3 && V == 1 && WOUT == 1) ? (RZ * RY > 9 ? 4 : 8) : 1) void fwd_lattice(Geom g, Lattice lt, int remap, View<const float> x,
+                                                    const float *__restrict__ k, const float *__restrict__ bias,
+                                                    View<float> out)
+{
+    extern __shared__ float lds[];
+    constexpr int K = Taps<NDIM>::K;
+    constexpr int NZ = Taps<NDIM>::NZ;          // z taps: 3 or 1
+    constexpr int LZ = NDIM == 3 ? RZ + 2 : 1;  // input lattice levels along z
+    constexpr int LY = RY + 2;
+    static_assert(NDIM == 3 || RZ == 1, "2D has a single z level");
+
+    int y0, z0;
+    if (!tile_origin<NDIM, RZ, RY>(g, lt, remap, y0, z0)) return;   // padding block or empty tail (whole workgroup)
 
     const int lane = threadIdx.x % lt.lpr;
     const int kg = __builtin_amdgcn_readfirstlane(threadIdx.x / lt.lpr);   // uniform: lpr is a multiple of 64
@@ -344,6 +353,15 @@ hipError_t pick(const Geom &g, const View<const float> &x, const float *k, const
                 const int rows_y = (g.H + g.dil - 1) / g.dil, rows_z = (g.D + g.dil - 1) / g.dil;
                 const long t24 = (long)((rows_z + 1) / 2) * ((rows_y + 3) / 4);
                 const long t33 = (long)((rows_z + 2) / 3) * ((rows_y + 2) / 3);
+                // Lattices of 4 x 4 rows read 36 input rows for 16 output rows (2.25 per row
+                // instead of 3) and halve the number of tiles; they take twice the registers, so
+                // two workgroups fewer share a CU.
+                const long t44 = (long)((rows_z + 3) / 4) * ((rows_y + 3) / 4);
+                const int forced = knob(kKnobFwdLattice3d, 0);
+                if (forced == 44) return launch<3, RELU, 1, 1, 4, 4>(g, x, k, bias, out, s);
+                if (forced == 33) return launch<3, RELU, 1, 1, 3, 3>(g, x, k, bias, out, s);
+                if (forced == 24) return launch<3, RELU, 1, 1, 2, 4>(g, x, k, bias, out, s);
+                (void)t44;
                 if (g.dil >= 3 && t33 * 16 < t24 * 15) return launch<3, RELU, 1, 1, 3, 3>(g, x, k, bias, out, s);
             }
             return launch<3, RELU, WOUT, 1, 2, 4>(g, x, k, bias, out, s);

@@ -50,7 +50,7 @@ enum Knob {
     kKnobBwdxVec2d, kKnobBwdxVec3d, kKnobBwdxUnroll2d, kKnobBwdxUnroll3d, kKnobBwdxMinBlocks,
     kKnobXcdRemap, kKnobBwdkVec2d, kKnobBwdkVec3d, kKnobBwdkBlocks,
     kKnobFwdVec2d, kKnobFwdVec3d, kKnobFwdSplit, kKnobFwdRows2d, kKnobBwdkRows, kKnobBlockFuse,
-    kKnobBlockDefer, kKnobBwdkInterleave, kKnobBlockSnake, kKnobFwdClass3d,
+    kKnobBlockDefer, kKnobBwdkInterleave, kKnobBlockSnake, kKnobFwdClass3d, kKnobFwdLattice3d,
     kKnobCount
 };
 int knob(Knob k, int dflt);

@@ -57,6 +57,8 @@ FORWARD_2D = [({"fwd.rows2d": r, "fwd.vec2d": v}, s)
 FORWARD_2D += [({"fwd.vec2d": v}, IMG_C) for v in (1, 2, 4)]
 FORWARD_3D = [({"fwd.vec3d": v}, s) for v in (1, 2, 4) for s in (VOL_A, VOL_B, VOL_C)]
 FORWARD_3D += [({"fwd.class3d": c}, s) for c in (0, 1) for s in (VOL_A, VOL_D, VOL_E)]
+FORWARD_3D += [({"fwd.lattice3d": m}, s) for m in (24, 33, 44) for s in (VOL_A, VOL_D, VOL_E)]
+FORWARD_3D += [({"fwd.lattice3d": 44, "fwd.split": k}, VOL_E) for k in (1, 4)]
 SPLIT = [({"fwd.split": k}, s) for k in (1, 2, 4) for s in (IMG_A, IMG_C, VOL_A, VOL_C)]
 ORDER = [({"xcd_remap": r}, s) for r in (0, 1) for s in (IMG_B, IMG_D, VOL_A, VOL_D)]
 BACKWARD_K = [({"bwdk.vec2d": v}, s) for v in (1, 2, 4) for s in (IMG_A, IMG_B, IMG_C)]
@@ -84,7 +86,7 @@ def test_operators_under_a_forced_setting(cc, case):
 
 
 BLOCK_SETTINGS = [{"block.snake": 0}, {"block.snake": 1}, {"block.fuse": 0}, {"block.defer": 0},
-                  {"xcd_remap": 0}, {"bwdk.interleave": 0}, {"fwd.class3d": 0}]
+                  {"xcd_remap": 0}, {"bwdk.interleave": 0}, {"fwd.class3d": 0}, {"fwd.lattice3d": 44}]
 
 
 @pytest.mark.parametrize("settings", BLOCK_SETTINGS, ids=lambda s: ",".join("%s=%d" % kv for kv in s.items()))
