@@ -293,6 +293,34 @@ int msd_final_backward(int dtype, int64_t batch, int64_t c_in, int64_t c_out, in
                        void *workspace, int64_t workspace_bytes, void *stream);
 
 /*
+ * Final layer, loss and the gradient of the loss in one pass over the stack: what the
+ * reference's models run as Conv1d [+ the 1x1 output scaling, folded into weight and bias by
+ * the caller] [+ LogSoftmax] + MSELoss / L1Loss / NLLLoss (msd_module.py:60-88,
+ * msd_model.py:220-223, msd_regression_model.py:5, msd_segmentation_model.py:61-68), all with
+ * the default 'mean' reduction.  c_out <= 8.
+ *   output       MSE, L1: bias + weight . input;  NLL: its log-softmax over the output channels
+ *   loss         one element of `dtype` in device memory
+ *   grad_output  d loss / d (bias + weight . input), same shape as output: handing it to
+ *                msd_final_backward (input, grad_weight, grad_bias NULL) gives the gradient of
+ *                the stack without reading the stack again
+ *   grad_weight, grad_bias   OVERWRITTEN with the layer's parameter gradients (both NULL: skipped)
+ * target: MSE, L1: values laid out like output (element strides given); NLL: int64 labels in
+ * [0, c_out), one per voxel, target_batch_stride in labels, target_channel_stride ignored.
+ * Workspace: msd_final_workspace_bytes.  Sums are reduced in a fixed order.
+ */
+#define MSD_LOSS_MSE 0
+#define MSD_LOSS_L1 1
+#define MSD_LOSS_NLL 2
+int msd_final_forward_loss(int dtype, int loss_kind, int64_t batch, int64_t c_in, int64_t c_out, int64_t nvox,
+                           const void *input, int64_t input_batch_stride, int64_t input_channel_stride,
+                           const void *weight, const void *bias,
+                           const void *target, int64_t target_batch_stride, int64_t target_channel_stride,
+                           void *output, int64_t output_batch_stride, int64_t output_channel_stride,
+                           void *grad_output, int64_t grad_output_batch_stride, int64_t grad_output_channel_stride,
+                           void *grad_weight, void *grad_bias, void *loss,
+                           void *workspace, int64_t workspace_bytes, void *stream);
+
+/*
  * Kernel timing for benchmarks.  While enabled, every operator call is bracketed by
  * HIP events recorded on its launch stream; inside the block calls consecutive launches
  * of one class share one pair of events (a pair per launch would add its own few

@@ -11,6 +11,7 @@ ABI_VERSION = 1
 
 MSD_F32, MSD_F64 = 0, 1
 MSD_OK, MSD_ERR_INVALID, MSD_ERR_HIP, MSD_ERR_WORKSPACE = 0, 1, 2, 3
+LOSS_MSE, LOSS_L1, LOSS_NLL = 0, 1, 2
 STATIC_SCRATCH_BYTES = 32 * 1024 * 1024   # MSD_STATIC_SCRATCH_BYTES of the header
 
 _c_int = ctypes.c_int
@@ -54,6 +55,9 @@ PROTOTYPES = {
                                    _ptr, _c_i64, _c_i64, _ptr]),
     "msd_final_backward": (_c_int, [_c_int, _c_i64, _c_i64, _c_i64, _c_i64, _ptr, _c_i64, _c_i64, _ptr, _c_i64, _c_i64,
                                     _ptr, _ptr, _c_i64, _c_i64, _ptr, _ptr] + _WS + [_ptr]),
+    "msd_final_forward_loss": (_c_int, [_c_int, _c_int, _c_i64, _c_i64, _c_i64, _c_i64, _ptr, _c_i64, _c_i64, _ptr, _ptr,
+                                        _ptr, _c_i64, _c_i64, _ptr, _c_i64, _c_i64, _ptr, _c_i64, _c_i64, _ptr, _ptr,
+                                        _ptr] + _WS + [_ptr]),
     "msd_profile_enable": (_c_int, [_c_int]),
     "msd_profile_read": (_c_int, [ctypes.POINTER(ctypes.c_double), _i64p]),
 }

@@ -996,6 +996,48 @@ int msd_final_backward(int dtype, int64_t batch, int64_t c_in, int64_t c_out, in
     return e == hipSuccess ? MSD_OK : hip_fail(fn, e);
 }
 
+int msd_final_forward_loss(int dtype, int loss_kind, int64_t batch, int64_t c_in, int64_t c_out, int64_t nvox,
+                           const void *input, int64_t input_batch_stride, int64_t input_channel_stride,
+                           const void *weight, const void *bias, const void *target, int64_t target_batch_stride,
+                           int64_t target_channel_stride, void *output, int64_t output_batch_stride,
+                           int64_t output_channel_stride, void *grad_output, int64_t grad_output_batch_stride,
+                           int64_t grad_output_channel_stride, void *grad_weight, void *grad_bias, void *loss,
+                           void *workspace, int64_t workspace_bytes, void *stream)
+{
+    const char *fn = "final_forward_loss";
+    MSD_TRY(check_final(fn, dtype, batch, c_in, c_out, nvox));
+    if (loss_kind < MSD_LOSS_MSE || loss_kind > MSD_LOSS_NLL)
+        return fail(MSD_ERR_INVALID, "%s: loss_kind must be MSD_LOSS_MSE, MSD_LOSS_L1 or MSD_LOSS_NLL", fn);
+    if (c_out > 8) return fail(MSD_ERR_INVALID, "%s: at most 8 output channels", fn);
+    if (!input || !weight || !target || !output || !grad_output || !loss)
+        return fail(MSD_ERR_INVALID, "%s: NULL argument", fn);
+    if (input_batch_stride < 0 || input_channel_stride < 0 || target_batch_stride < 0 || target_channel_stride < 0 ||
+        output_batch_stride < 0 || output_channel_stride < 0 || grad_output_batch_stride < 0 ||
+        grad_output_channel_stride < 0)
+        return fail(MSD_ERR_INVALID, "%s: negative stride", fn);
+    const int64_t need = msd_final_workspace_bytes(dtype, batch, c_in, c_out, nvox);
+    if (!workspace || workspace_bytes < need)
+        return fail(MSD_ERR_WORKSPACE, "%s: workspace of %lld bytes needed, %lld given", fn, (long long)need,
+                    (long long)(workspace ? workspace_bytes : 0));
+    const hipError_t e =
+        dtype == MSD_F32
+            ? msd::final_forward_loss<float>(loss_kind, batch, (int)c_in, (int)c_out, nvox, (const float *)input,
+                                             input_batch_stride, input_channel_stride, (const float *)weight,
+                                             (const float *)bias, target, target_batch_stride, target_channel_stride,
+                                             (float *)output, output_batch_stride, output_channel_stride,
+                                             (float *)grad_output, grad_output_batch_stride,
+                                             grad_output_channel_stride, (float *)grad_weight, (float *)grad_bias,
+                                             (float *)loss, (float *)workspace, (hipStream_t)stream)
+            : msd::final_forward_loss<double>(loss_kind, batch, (int)c_in, (int)c_out, nvox, (const double *)input,
+                                              input_batch_stride, input_channel_stride, (const double *)weight,
+                                              (const double *)bias, target, target_batch_stride,
+                                              target_channel_stride, (double *)output, output_batch_stride,
+                                              output_channel_stride, (double *)grad_output, grad_output_batch_stride,
+                                              grad_output_channel_stride, (double *)grad_weight, (double *)grad_bias,
+                                              (double *)loss, (double *)workspace, (hipStream_t)stream);
+    return e == hipSuccess ? MSD_OK : hip_fail(fn, e);
+}
+
 int msd_profile_enable(int on)
 {
     g_profile.on = on != 0;

@@ -166,11 +166,134 @@ __global__ __launch_bounds__(kFinalThreads) void final_backward_kernel(int64_t n
     }
 }
 
+// Final layer, loss and the loss's gradient in one pass over the stack:
+//     out = bias + w . x              (NLL: out = log_softmax over the output channels of that)
+//     loss = mean of (out - t)^2 | |out - t| | -out[label]
+//     g = d loss / d (bias + w . x)   written to gout
+// and, for the layer's own parameters, the partial sums of  sum_n g[o][n] * x[c][n]  and
+// sum_n g[o][n]  (a second walk over the channels of the same voxels, which the caches
+// serve): everything the backward pass needs from the stack, so that it does not have to read
+// the stack again.  Columns of `part`: (o, c) -> o * C + c, then c_out bias columns, then the loss.
+template <typename T, int V, int MAXO, int KIND>
+__global__ __launch_bounds__(kFinalThreads) void final_forward_loss_kernel(
+    int64_t nvec, int C, int c_out, const T *__restrict__ x, int64_t xsb, int64_t xsc, const T *__restrict__ w,
+    const T *__restrict__ bias, const void *__restrict__ target, int64_t tsb, int64_t tsc, T *__restrict__ out,
+    int64_t osb, int64_t osc, T *__restrict__ gout, int64_t gsb, int64_t gsc, T inv_n, int want_sums,
+    T *__restrict__ part, int64_t rows)
+{
+    const int64_t i = (int64_t)blockIdx.x * kFinalThreads + threadIdx.x;
+    const bool active = i < nvec;
+    const int64_t ic = active ? i : nvec - 1;     // lanes past the end work on a valid voxel and contribute zeros
+    const int b = blockIdx.y;
+    const int lane = threadIdx.x % kWave;
+    const int64_t row = ((int64_t)b * gridDim.x + blockIdx.x) * (kFinalThreads / kWave) + threadIdx.x / kWave;
+    const T *xp = x + (int64_t)b * xsb + ic * V;
+    T acc[MAXO][V];
+#pragma unroll
+    for (int o = 0; o < MAXO; o++)
+#pragma unroll
+        for (int e = 0; e < V; e++) acc[o][e] = T(0);
+#pragma unroll 4
+    for (int c = 0; c < C; c++) {
+        T v[V];
+        load_elems<T, V>(xp + (int64_t)c * xsc, v);
+#pragma unroll
+        for (int o = 0; o < MAXO; o++) {
+            const T wv = w[(int64_t)min(o, c_out - 1) * C + c];
+#pragma unroll
+            for (int e = 0; e < V; e++) acc[o][e] += wv * v[e];
+        }
+    }
+    T g[MAXO][V];
+    T lsum = T(0);
+    if constexpr (KIND == 2) {
+        // log-softmax over the output channels, then the negative log-likelihood of the label
+        const int64_t *lab = static_cast<const int64_t *>(target) + (int64_t)b * tsb + ic * V;
+#pragma unroll
+        for (int e = 0; e < V; e++) {
+            T m = acc[0][e] + (bias ? bias[0] : T(0));
+#pragma unroll
+            for (int o = 0; o < MAXO; o++) {
+                acc[o][e] += bias && o < c_out ? bias[o] : T(0);
+                if (o < c_out) m = acc[o][e] > m ? acc[o][e] : m;
+            }
+            T se = T(0);
+#pragma unroll
+            for (int o = 0; o < MAXO; o++)
+                if (o < c_out) se += exp(acc[o][e] - m);
+            const T lse = m + log(se);
+            const int64_t t = lab[e];
+#pragma unroll
+            for (int o = 0; o < MAXO; o++) {
+                acc[o][e] -= lse;                             // log-probability
+                const T pr = o < c_out ? exp(acc[o][e]) : T(0);
+                g[o][e] = active && o < c_out ? (pr - (t == o ? T(1) : T(0))) * inv_n : T(0);
+                if (active && t == o) lsum -= acc[o][e];
+            }
+        }
+    } else {
+#pragma unroll
+        for (int o = 0; o < MAXO; o++) {
+            const bool keep = active && o < c_out;
+            T t[V];
+            load_elems<T, V>(static_cast<const T *>(target) + (int64_t)b * tsb + (int64_t)min(o, c_out - 1) * tsc + ic * V,
+                             t);
+            const T bv = bias && o < c_out ? bias[o] : T(0);
+#pragma unroll
+            for (int e = 0; e < V; e++) {
+                acc[o][e] += bv;
+                const T diff = acc[o][e] - t[e];
+                if (KIND == 0) {
+                    g[o][e] = keep ? T(2) * diff * inv_n : T(0);
+                    lsum += keep ? diff * diff : T(0);
+                } else {
+                    g[o][e] = keep ? (diff > T(0) ? inv_n : (diff < T(0) ? -inv_n : T(0))) : T(0);
+                    lsum += keep ? (diff < T(0) ? -diff : diff) : T(0);
+                }
+            }
+        }
+    }
+    if (active) {
+#pragma unroll
+        for (int o = 0; o < MAXO; o++) {
+            if (o >= c_out) break;
+            store_elems<T, V>(out + (int64_t)b * osb + (int64_t)o * osc + i * V, acc[o]);
+            store_elems<T, V>(gout + (int64_t)b * gsb + (int64_t)o * gsc + i * V, g[o]);
+        }
+    }
+    lsum = wave_sum(lsum * inv_n);
+    if (lane == 0) part[((int64_t)c_out * C + c_out) * rows + row] = lsum;
+    if (!want_sums) return;                                   // uniform
+#pragma unroll
+    for (int o = 0; o < MAXO; o++) {
+        T sb = T(0);
+#pragma unroll
+        for (int e = 0; e < V; e++) sb += g[o][e];
+        sb = wave_sum(sb);
+        if (lane == 0 && o < c_out) part[((int64_t)c_out * C + o) * rows + row] = sb;
+    }
+#pragma unroll 2
+    for (int c = 0; c < C; c++) {
+        T v[V];
+        load_elems<T, V>(xp + (int64_t)c * xsc, v);
+#pragma unroll
+        for (int o = 0; o < MAXO; o++) {
+            T sw = T(0);
+#pragma unroll
+            for (int e = 0; e < V; e++) sw += g[o][e] * v[e];
+            sw = wave_sum(sw);
+            if (lane == 0 && o < c_out) part[((int64_t)o * C + c) * rows + row] = sw;
+        }
+    }
+}
+
 // One workgroup per column: thread t adds rows t, t + 256, ... in order, a fixed shuffle tree
 // adds the lanes of each wave and the four wave sums are added in order.
+// Columns [0, nw) go to gw, [nw, nw + nb) to gb, a last one (if any) to `loss`.
 template <typename T>
 __global__ __launch_bounds__(256) void final_reduce_kernel(const T *__restrict__ part, int64_t rows, int64_t nw,
-                                                           int64_t ncols, T *__restrict__ gw, T *__restrict__ gb)
+                                                           int64_t nb, T *__restrict__ gw, T *__restrict__ gb,
+                                                           T *__restrict__ loss)
 {
     __shared__ T wave_sum[256 / kWave];
     const int64_t col = blockIdx.x;
@@ -186,8 +309,10 @@ __global__ __launch_bounds__(256) void final_reduce_kernel(const T *__restrict__
         for (int w = 1; w < 256 / kWave; w++) total += wave_sum[w];
         if (col < nw) {
             if (gw) gw[col] = total;
-        } else if (gb) {
-            gb[col - nw] = total;
+        } else if (col < nw + nb) {
+            if (gb) gb[col - nw] = total;
+        } else if (loss) {
+            *loss = total;
         }
     }
 }
@@ -220,7 +345,7 @@ int64_t final_rows(int64_t batch, int64_t nvox)
 
 int64_t final_workspace_elems(int64_t batch, int64_t c_in, int64_t c_out, int64_t nvox)
 {
-    return (c_out * c_in + c_out) * final_rows(batch, nvox);
+    return (c_out * c_in + c_out + 1) * final_rows(batch, nvox);   // weight, bias and loss columns
 }
 
 template <typename T>
@@ -278,9 +403,71 @@ hipError_t final_backward(int64_t batch, int c_in, int c_out, int64_t nvox, cons
     }
     if (!ws) return hipSuccess;
     const int64_t nw = (int64_t)c_out * c_in, ncols = nw + c_out;
-    hipLaunchKernelGGL(final_reduce_kernel<T>, dim3((unsigned)ncols), dim3(256), 0, s, ws, rows, nw, ncols, gw, gb);
+    hipLaunchKernelGGL(final_reduce_kernel<T>, dim3((unsigned)ncols), dim3(256), 0, s, ws, rows, nw, (int64_t)c_out, gw,
+                       gb, (T *)nullptr);
     return hipGetLastError();
 }
+
+template <typename T>
+hipError_t final_forward_loss(int kind, int64_t batch, int c_in, int c_out, int64_t nvox, const T *x, int64_t xsb,
+                              int64_t xsc, const T *w, const T *bias, const void *target, int64_t tsb, int64_t tsc,
+                              T *out, int64_t osb, int64_t osc, T *gout, int64_t gsb, int64_t gsc, T *gw, T *gb,
+                              T *loss, T *ws, hipStream_t s)
+{
+    // labels are one int64 per voxel: no vector width to match
+    const int V = kind == 2 ? final_vec<T>(nvox, {{x, {xsb, xsc}}, {out, {osb, osc}}, {gout, {gsb, gsc}}})
+                            : final_vec<T>(nvox, {{x, {xsb, xsc}}, {out, {osb, osc}}, {gout, {gsb, gsc}},
+                                                  {target, {tsb, tsc}}});
+    const int64_t nvec = nvox / V;
+    const dim3 grid((unsigned)((nvec + kFinalThreads - 1) / kFinalThreads), (unsigned)batch, 1);
+    const int64_t rows = (int64_t)grid.x * batch * (kFinalThreads / kWave);
+    const int64_t terms = kind == 2 ? batch * nvox : batch * nvox * (int64_t)c_out;
+    const T inv_n = T(1) / T(terms);
+    const int want = gw || gb;
+    const int mo = c_out > 4 ? 8 : (c_out > 2 ? 4 : (c_out > 1 ? 2 : 1));
+#define MSD_FINAL_LOSS(VV, OO, KK)                                                                                  \
+    hipLaunchKernelGGL((final_forward_loss_kernel<T, VV, OO, KK>), grid, dim3(kFinalThreads), 0, s, nvec, c_in, c_out, \
+                       x, xsb, xsc, w, bias, target, tsb, tsc, out, osb, osc, gout, gsb, gsc, inv_n, want, ws, rows)
+#define MSD_FINAL_LOSS_O(VV, KK)                                                                        \
+    do {                                                                                                \
+        if (mo == 8) MSD_FINAL_LOSS(VV, 8, KK); else if (mo == 4) MSD_FINAL_LOSS(VV, 4, KK);            \
+        else if (mo == 2) MSD_FINAL_LOSS(VV, 2, KK); else MSD_FINAL_LOSS(VV, 1, KK);                    \
+    } while (0)
+#define MSD_FINAL_LOSS_K(VV)                                                                            \
+    do {                                                                                                \
+        if (kind == 0) MSD_FINAL_LOSS_O(VV, 0); else if (kind == 1) MSD_FINAL_LOSS_O(VV, 1); else MSD_FINAL_LOSS_O(VV, 2); \
+    } while (0)
+    if (V == 1) {
+        MSD_FINAL_LOSS_K(1);
+    } else {
+        constexpr int W = wide_vec<T>();
+        MSD_FINAL_LOSS_K(W);
+    }
+#undef MSD_FINAL_LOSS_K
+#undef MSD_FINAL_LOSS_O
+#undef MSD_FINAL_LOSS
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    const int64_t nw = (int64_t)c_out * c_in;
+    if (want) {
+        hipLaunchKernelGGL(final_reduce_kernel<T>, dim3((unsigned)(nw + c_out + 1)), dim3(256), 0, s, ws, rows, nw,
+                           (int64_t)c_out, gw, gb, loss);
+    } else {
+        // only the loss column was written
+        hipLaunchKernelGGL(final_reduce_kernel<T>, dim3(1), dim3(256), 0, s, ws + (nw + c_out) * rows, rows, (int64_t)0,
+                           (int64_t)0, (T *)nullptr, (T *)nullptr, loss);
+    }
+    return hipGetLastError();
+}
+
+template hipError_t final_forward_loss<float>(int, int64_t, int, int, int64_t, const float *, int64_t, int64_t,
+                                              const float *, const float *, const void *, int64_t, int64_t, float *,
+                                              int64_t, int64_t, float *, int64_t, int64_t, float *, float *, float *,
+                                              float *, hipStream_t);
+template hipError_t final_forward_loss<double>(int, int64_t, int, int, int64_t, const double *, int64_t, int64_t,
+                                               const double *, const double *, const void *, int64_t, int64_t,
+                                               double *, int64_t, int64_t, double *, int64_t, int64_t, double *,
+                                               double *, double *, double *, hipStream_t);
 
 template hipError_t final_forward<float>(int64_t, int, int, int64_t, const float *, int64_t, int64_t, const float *,
                                          const float *, float *, int64_t, int64_t, hipStream_t);

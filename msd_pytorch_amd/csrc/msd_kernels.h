@@ -45,6 +45,16 @@ hipError_t final_backward(int64_t batch, int c_in, int c_out, int64_t nvox, cons
                           const T *go, int64_t gsb, int64_t gsc, const T *w, T *gx, int64_t gxsb, int64_t gxsc,
                           T *gw, T *gb, T *ws, hipStream_t s);
 
+// Final layer + loss + the loss's gradient in one pass (kind 0: mean squared error, 1: mean
+// absolute error, 2: log-softmax over the output channels + negative log-likelihood of int64
+// labels); c_out <= 8.  Writes out, gout = d loss / d (layer output), the scalar loss and (unless
+// both null) gw, gb.  ws as for final_backward.
+template <typename T>
+hipError_t final_forward_loss(int kind, int64_t batch, int c_in, int c_out, int64_t nvox, const T *x, int64_t xsb,
+                              int64_t xsc, const T *w, const T *bias, const void *target, int64_t tsb, int64_t tsc,
+                              T *out, int64_t osb, int64_t osc, T *gout, int64_t gsb, int64_t gsc, T *gw, T *gb,
+                              T *loss, T *ws, hipStream_t s);
+
 // Launch-shape knobs (msd_set_tuning in the C ABI).  A value < 0 means "library default".
 enum Knob {
     kKnobBwdxVec2d, kKnobBwdxVec3d, kKnobBwdxUnroll2d, kKnobBwdxUnroll3d, kKnobBwdxMinBlocks,

@@ -539,3 +539,63 @@ def final_backward(input, grad_output, weight, grad_input, grad_weight, grad_bia
     _call("msd_final_backward", input.device, _DTYPES[input.dtype], input.shape[0], c_in, c_out, nvox, ptr(input), isb,
           isc, ptr(grad_output), gsb, gsc, ptr(weight), ptr(grad_input), xsb, xsc, ptr(grad_weight), ptr(grad_bias),
           ptr(ws), int(need), _stream(input))
+
+
+LOSS_KINDS = {"mse": _native.LOSS_MSE, "l1": _native.LOSS_L1, "nll": _native.LOSS_NLL}
+
+
+def final_forward_loss(input, weight, bias, kind, target, grad_weight=None, grad_bias=None):
+    """Final layer, loss and the loss's gradient in one pass over ``input`` (B, C, *spatial):
+    ``kind`` "mse" / "l1" (target shaped like the output) or "nll" (log-softmax over the output
+    channels, int64 labels (B, *spatial)); 'mean' reduction; at most 8 output channels.
+    Returns (output, loss, grad_output) with grad_output = d loss / d (bias + weight . input);
+    ``grad_weight`` / ``grad_bias`` (or None) are overwritten with the layer's parameter
+    gradients."""
+    fn = "final_forward_loss"
+    if kind not in LOSS_KINDS:
+        raise ValueError(f"{fn}: kind must be one of {sorted(LOSS_KINDS)}")
+    named = [("input", input), ("weight", weight), ("target", target)]
+    named += [(n, t) for n, t in (("bias", bias), ("grad_weight", grad_weight), ("grad_bias", grad_bias))
+              if t is not None]
+    _check_same_gpu(fn, named)
+    _check_same_type(fn, [(n, t) for n, t in named if n != "target" or kind != "nll"])
+    c_out, c_in = weight.shape[0], weight.shape[1]
+    if weight.numel() != c_out * c_in or not weight.is_contiguous():
+        _fail(fn, "Expected weight to be contiguous and shaped (c_out, c_in[, 1])")
+    if c_out > 8:
+        _fail(fn, "at most 8 output channels")
+    if input.shape[1] != c_in:
+        _fail(fn, "Kernel shape does not match input channels. ")
+    if not final_layer_supported(input):
+        _fail(fn, "Expected channel planes to be contiguous")
+    for name, t, n in (("bias", bias, c_out), ("grad_bias", grad_bias, c_out), ("grad_weight", grad_weight, c_out * c_in)):
+        if t is not None and (t.numel() != n or not t.is_contiguous()):
+            _fail(fn, f"Expected {name} to be contiguous with {n} elements")
+    out_shape = (input.shape[0], c_out, *input.shape[2:])
+    nvox, isb, isc = _flat_strides(input)
+    if kind == "nll":
+        if target.dtype != torch.int64 or tuple(target.shape) != (input.shape[0], *input.shape[2:]) \
+                or not target.is_contiguous():
+            _fail(fn, "Expected contiguous int64 labels shaped (B, *spatial)")
+        tsb, tsc = nvox, 0
+    else:
+        if tuple(target.shape) != out_shape or not final_layer_supported(target):
+            _fail(fn, "Expected a target shaped like the output with contiguous channel planes")
+        _, tsb, tsc = _flat_strides(target)
+    output = torch.empty(out_shape, dtype=input.dtype, device=input.device)
+    grad_output = torch.empty_like(output)
+    loss = torch.empty((), dtype=input.dtype, device=input.device)
+    _, osb, osc = _flat_strides(output)
+    lib = _native.load()
+    need = lib.msd_final_workspace_bytes(_DTYPES[input.dtype], input.shape[0], c_in, c_out, nvox)
+    if need < 0:
+        _fail(fn, _native.last_error())
+    ws = torch.empty(max(int(need), 8), dtype=torch.uint8, device=input.device)
+
+    def ptr(t):
+        return ctypes.c_void_p(t.data_ptr() if t is not None else 0)
+
+    _call("msd_final_forward_loss", input.device, _DTYPES[input.dtype], LOSS_KINDS[kind], input.shape[0], c_in, c_out,
+          nvox, ptr(input), isb, isc, ptr(weight), ptr(bias), ptr(target), tsb, tsc, ptr(output), osb, osc,
+          ptr(grad_output), osb, osc, ptr(grad_weight), ptr(grad_bias), ptr(loss), ptr(ws), int(need), _stream(input))
+    return output, loss, grad_output

@@ -201,8 +201,34 @@ class MSDModel:
             self.set_target(target)
         self.output = None
         self.loss = None
+        fused = self._fused_forward_loss() if self.fuse_loss else None
+        if fused is not None:
+            self.loss, self.output = fused
+            return
         self.output = self.net(self.input)
         self.loss = self.criterion(self.output, self.target)
+
+    # Loss computed in the pass of the final layer (MSDModule.forward_loss) where the model has
+    # the standard structure; set to False to run network and criterion as separate modules.
+    fuse_loss = True
+
+    def _loss_kind(self):
+        """"mse", "l1" or "nll" when the criterion is torch's with default settings, else None."""
+        c = self.criterion
+        if getattr(c, "reduction", None) != "mean":
+            return None
+        if type(c) is nn.MSELoss:
+            return "mse"
+        if type(c) is nn.L1Loss:
+            return "l1"
+        if type(c) is nn.NLLLoss and c.weight is None and c.ignore_index == -100:
+            return "nll"
+        return None
+
+    def _fused_forward_loss(self):
+        """(loss, output) through the fused node, or None when the model is not the plain
+        scale_in -> msd [-> scale_out | -> LogSoftmax] -> criterion chain on the GPU."""
+        return None
 
     def forward(self, input=None, target=None):
         """Loss of one (input, target) pair; arguments left out keep their last value."""

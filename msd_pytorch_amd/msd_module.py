@@ -91,6 +91,62 @@ class MSDNetFunction(torch.autograd.Function):
         return (grad_input, None, grad_bias, grad_fw, grad_fb, *grad_weights)
 
 
+class MSDNetLossFunction(torch.autograd.Function):
+    """Dense block, final layer, an optional frozen 1x1 output scaling and the loss as ONE
+    autograd node:
+    ``(input, dilations, bias, final_weight, final_bias, scale_weight, scale_bias, target, kind,
+    *weights) -> (loss, output)``.
+
+    ``kind`` is "mse", "l1" (output = scale(final(stack)), loss against ``target``) or "nll"
+    (output = log_softmax(final(stack)), int64 labels).  The pass that computes the final layer
+    also computes the loss, its gradient with respect to the layer's output and the layer's own
+    parameter gradients, so the backward pass starts from a tensor of c_out channels and never
+    reads the stack for the final layer again.  ``output`` is returned for the caller's use and
+    is not differentiable; the scaling layer's parameters get no gradient (they are frozen in
+    the models, msd_model.py:8-45)."""
+
+    @staticmethod
+    def forward(ctx, input, dilations, bias, final_weight, final_bias, scale_weight, scale_bias, target, kind,
+                *weights):
+        stack = block_stack_forward(input, dilations, bias, weights)
+        c_out = final_weight.shape[0]
+        fw = final_weight.view(c_out, -1)
+        if scale_weight is not None:
+            sw = scale_weight.view(c_out, c_out)
+            w_eff = (sw @ fw).contiguous()
+            b_eff = sw @ final_bias + scale_bias
+        else:
+            sw, w_eff, b_eff = None, fw.contiguous(), final_bias
+        need_fw, need_fb = ctx.needs_input_grad[3], ctx.needs_input_grad[4]
+        g_w = torch.empty_like(w_eff) if need_fw or need_fb else None
+        g_b = torch.empty_like(b_eff) if need_fw or need_fb else None
+        output, loss, grad_out = cc.final_forward_loss(stack, w_eff, b_eff, kind, target, g_w, g_b)
+        ctx.dilations = tuple(dilations)
+        ctx.save_for_backward(bias, stack, w_eff, grad_out, g_w, g_b, sw, *weights)
+        ctx.final_shape = final_weight.shape
+        ctx.mark_non_differentiable(output)
+        return loss, output
+
+    @staticmethod
+    def backward(ctx, grad_loss, _grad_output):
+        bias, stack, w_eff, grad_out, g_w, g_b, sw, *weights = ctx.saved_tensors
+        need_input, _, need_bias, need_fw, need_fb, *rest = ctx.needs_input_grad
+        need_weights = rest[4:]
+        grad_fw = grad_fb = None
+        if need_fw or need_fb:
+            # chain through the frozen scaling layer: W_eff = S W, b_eff = S b + t
+            gw, gb = (sw.t() @ g_w, sw.t() @ g_b) if sw is not None else (g_w, g_b)
+            grad_fw = (gw * grad_loss).view(ctx.final_shape) if need_fw else None
+            grad_fb = gb * grad_loss if need_fb else None
+        grad_input, grad_bias, grad_weights = (None, None, [None] * len(weights))
+        if need_input or need_bias or any(need_weights):
+            grads = torch.empty_like(stack)
+            cc.final_backward(None, grad_out * grad_loss, w_eff, grads, None, None)
+            grad_input, grad_bias, grad_weights = block_stack_backward(
+                stack, grads, ctx.dilations, bias, weights, need_input, need_bias, need_weights)
+        return (grad_input, None, grad_bias, grad_fw, grad_fb, None, None, None, None, *grad_weights)
+
+
 class MSDFinalLayer(torch.nn.Module):
     """1x1 convolution over the whole channel stack, zero-initialised.
 
@@ -167,3 +223,32 @@ class MSDModule(torch.nn.Module):
             weights = (getattr(block, f"weight{i}") for i in range(len(block.weights)))
             return MSDNetFunction.apply(input, block.dilations, block.bias, linear.weight, linear.bias, *weights)
         return self.final_layer(self.msd_block(input))
+
+    def forward_loss(self, input, target, kind, scale=None):
+        """(loss, output) of the network followed by an optional frozen 1x1 ``scale`` layer and
+        the loss ``kind`` ("mse", "l1", "nll"), as one autograd node (MSDNetLossFunction), or
+        None where that node does not apply (the caller then runs the modules one by one):
+        CPU tensors, more than 8 output channels, hooks on the sub-modules, a scaling layer
+        that is being trained."""
+        linear = self.final_layer.linear
+        if not (cc.final_layer_supported(input) and input.dim() in (4, 5) and input.dtype == linear.weight.dtype
+                and linear.bias is not None and not self._hooked() and self.c_out <= 8 and target.is_cuda):
+            return None
+        sw = sb = None
+        if scale is not None:
+            if scale.weight.requires_grad or scale.bias is None or scale.bias.requires_grad \
+                    or scale.weight.dtype != input.dtype or scale._forward_hooks or scale._forward_pre_hooks:
+                return None
+            sw, sb = scale.weight, scale.bias
+        if kind == "nll":
+            if target.dtype != torch.int64 or tuple(target.shape) != (input.shape[0], *input.shape[2:]):
+                return None
+            target = target.contiguous()
+        else:
+            if target.dtype != input.dtype or tuple(target.shape) != (input.shape[0], self.c_out, *input.shape[2:]) \
+                    or not cc.final_layer_supported(target):
+                return None
+        block = self.msd_block
+        weights = (getattr(block, f"weight{i}") for i in range(len(block.weights)))
+        return MSDNetLossFunction.apply(input, block.dilations, block.bias, linear.weight, linear.bias, sw, sb,
+                                        target, kind, *weights)

@@ -23,3 +23,10 @@ class MSDRegressionModel(MSDModel):
             self.net = nn.DataParallel(self.net)
         # only the MSD module is trained; the scaling layers are frozen
         self.init_optimizer(self.msd)
+
+    def _fused_forward_loss(self):
+        kind = self._loss_kind()
+        if kind is None or not isinstance(self.net, nn.Sequential) or len(self.net) != 3 \
+                or self.net[1] is not self.msd or self.net[2] is not self.scale_out:
+            return None
+        return self.msd.forward_loss(self.net[0](self.input), self.target, kind, scale=self.scale_out)

@@ -35,3 +35,12 @@ class MSDSegmentationModel(MSDModel):
                 f"Target invalid: expected values in range {[0, self.num_labels - 1]}, but got {[lo, hi]}")
         # NLLLoss takes (B, *spatial) class indices: drop the channel axis
         self.target = target.squeeze(1).cuda()
+
+    def _fused_forward_loss(self):
+        if self._loss_kind() != "nll" or not isinstance(self.net, nn.Sequential) or len(self.net) != 2:
+            return None
+        trained = self.net[1]
+        if not isinstance(trained, nn.Sequential) or len(trained) != 2 or trained[0] is not self.msd \
+                or type(trained[1]) is not nn.LogSoftmax or trained[1].dim != 1:
+            return None
+        return self.msd.forward_loss(self.net[0](self.input), self.target, "nll")

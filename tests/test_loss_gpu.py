@@ -1,0 +1,163 @@
+"""The final layer fused with the loss (msd_final_forward_loss) against torch in double
+precision: output, loss value, the gradient handed to the backward pass and the layer's
+parameter gradients, for the three losses of the reference's models (MSELoss and L1Loss of
+msd_regression_model.py:5, LogSoftmax + NLLLoss of msd_segmentation_model.py:61-68), and the
+models with and without the fused node.
+
+Tolerances: fp32 values 1e-5 and gradients 1e-4 relative to the largest reference magnitude;
+fp64 1e-11."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from cases import rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def reference(kind, x, w, b, target):
+    """torch, double precision: (output, loss, d loss / d pre-activation, grad_w, grad_b)."""
+    x, w, b = x.double(), w.double().requires_grad_(True), b.double().requires_grad_(True)
+    pre = torch.einsum("oc,bc...->bo...", w, x) + b.view(1, -1, *([1] * (x.dim() - 2)))
+    pre.retain_grad()
+    if kind == "nll":
+        out = F.log_softmax(pre, dim=1)
+        loss = F.nll_loss(out, target)
+    else:
+        out = pre
+        loss = F.mse_loss(out, target.double()) if kind == "mse" else F.l1_loss(out, target.double())
+    loss.backward()
+    return out.detach(), loss.detach(), pre.grad, w.grad, b.grad
+
+
+CASES = [
+    # (batch, c_in, c_out, spatial)
+    (1, 7, 1, (33, 64)),
+    (3, 12, 2, (17, 31)),          # odd plane size: one voxel per thread
+    (2, 5, 4, (6, 10, 12)),
+    (1, 21, 5, (40, 44)),
+    (2, 3, 8, (5, 6, 8)),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("kind", ["mse", "l1", "nll"])
+@pytest.mark.parametrize("batch,c_in,c_out,spatial", CASES)
+def test_fused_loss_matches_torch(batch, c_in, c_out, spatial, kind, dtype):
+    from msd_pytorch_amd import msd_custom_convolutions as cc
+    gen = torch.Generator().manual_seed(c_in * 100 + c_out)
+    # the input is a channel slice of a larger stack, as the dense block hands it over
+    stack = torch.randn(batch, c_in + 2, *spatial, generator=gen, dtype=dtype)
+    x = stack[:, :c_in]
+    w = torch.randn(c_out, c_in, generator=gen, dtype=dtype) * 0.3
+    b = torch.randn(c_out, generator=gen, dtype=dtype)
+    if kind == "nll":
+        target = torch.randint(0, c_out, (batch, *spatial), generator=gen)
+    else:
+        target = torch.randn(batch, c_out, *spatial, generator=gen, dtype=dtype)
+    want_out, want_loss, want_g, want_gw, want_gb = reference(kind, x, w, b, target)
+
+    xd = stack.cuda()[:, :c_in]
+    gw = torch.full((c_out, c_in), 7.0, dtype=dtype, device="cuda")      # overwritten, not accumulated into
+    gb = torch.full((c_out,), 7.0, dtype=dtype, device="cuda")
+    out, loss, g = cc.final_forward_loss(xd, w.cuda(), b.cuda(), kind, target.cuda(), gw, gb)
+    tv, tg = (1e-5, 1e-4) if dtype == torch.float32 else (1e-11, 1e-11)
+    assert rel_err(out, want_out) <= tv
+    assert abs(loss.item() - want_loss.item()) <= tv * max(abs(want_loss.item()), 1e-30)
+    assert rel_err(g, want_g) <= tg
+    assert rel_err(gw, want_gw) <= tg and rel_err(gb, want_gb) <= tg
+    # without parameter gradients: same values, and the stack gradient from g alone
+    out2, loss2, g2 = cc.final_forward_loss(xd, w.cuda(), b.cuda(), kind, target.cuda())
+    assert torch.equal(out2, out) and torch.equal(g2, g) and loss2.item() == loss.item()
+    gx = torch.empty(batch, c_in, *spatial, dtype=dtype, device="cuda")
+    cc.final_backward(None, g, w.cuda(), gx, None, None)
+    want_gx = torch.einsum("oc,bo...->bc...", w.double(), want_g)
+    assert rel_err(gx, want_gx) <= tg
+
+
+def test_fused_loss_rejects_what_it_does_not_take():
+    from msd_pytorch_amd import msd_custom_convolutions as cc
+    x = torch.zeros(1, 3, 8, 8, device="cuda")
+    with pytest.raises(RuntimeError, match="8 output channels"):
+        cc.final_forward_loss(x, torch.zeros(9, 3, device="cuda"), None, "mse", torch.zeros(1, 9, 8, 8, device="cuda"))
+    with pytest.raises(RuntimeError, match="int64 labels"):
+        cc.final_forward_loss(x, torch.zeros(2, 3, device="cuda"), None, "nll", torch.zeros(1, 8, 8, device="cuda"))
+    with pytest.raises(ValueError):
+        cc.final_forward_loss(x, torch.zeros(2, 3, device="cuda"), None, "huber", torch.zeros(1, 2, 8, 8, device="cuda"))
+
+
+def _grads(model):
+    return {n: p.grad.clone() for n, p in model.net.named_parameters() if p.grad is not None}
+
+
+@pytest.mark.parametrize("ndim,size", [(2, (40, 64)), (3, (8, 10, 32))])
+@pytest.mark.parametrize("loss", ["L2", "L1"])
+def test_regression_model_with_and_without_the_fused_loss(ndim, size, loss):
+    from msd_pytorch_amd import MSDRegressionModel
+    torch.manual_seed(3)
+    model = MSDRegressionModel(2, 3, 7, 1, loss=loss, ndim=ndim)
+    model.msd.final_layer.linear.weight.data.normal_(0, 0.1)
+    model.msd.final_layer.linear.bias.data.normal_(0, 0.1)
+    x = torch.rand(2, 2, *size)
+    t = torch.randn(2, 3, *size)
+    model.set_normalization([(x, t)])                      # non-trivial scaling layers
+    results = []
+    for fused in (True, False):
+        model.fuse_loss = fused
+        value = model.gradients(x, t)
+        results.append((value, model.output.clone(), _grads(model)))
+    (l1, o1, g1), (l0, o0, g0) = results
+    assert type(model.loss.grad_fn).__name__ != "MSDNetLossFunctionBackward"      # the last run was unfused
+    assert abs(l1 - l0) <= 1e-5 * abs(l0)
+    assert rel_err(o1, o0) <= 1e-5
+    assert set(g1) == set(g0) and len(g1) >= 9
+    for name in g0:
+        assert rel_err(g1[name], g0[name]) <= 1e-4, name
+    model.fuse_loss = True
+    model.forward(x, t)
+    assert type(model.loss.grad_fn).__name__ == "MSDNetLossFunctionBackward"
+
+
+@pytest.mark.parametrize("ndim,size", [(2, (40, 64)), (3, (8, 10, 32))])
+def test_segmentation_model_with_and_without_the_fused_loss(ndim, size):
+    from msd_pytorch_amd import MSDSegmentationModel
+    torch.manual_seed(4)
+    model = MSDSegmentationModel(1, 4, 6, 1, ndim=ndim)
+    model.msd.final_layer.linear.weight.data.normal_(0, 0.2)
+    x = torch.rand(2, 1, *size)
+    t = torch.randint(0, 4, (2, 1, *size))
+    results = []
+    for fused in (True, False):
+        model.fuse_loss = fused
+        value = model.gradients(x, t)
+        results.append((value, model.output.clone(), _grads(model)))
+    (l1, o1, g1), (l0, o0, g0) = results
+    assert abs(l1 - l0) <= 1e-5 * abs(l0)
+    assert rel_err(o1, o0) <= 1e-5
+    for name in g0:
+        assert rel_err(g1[name], g0[name]) <= 1e-4, name
+    # learning works through the fused node
+    model.fuse_loss = True
+    before = [p.detach().clone() for p in model.msd.parameters()]
+    first = model.learn(x, t)
+    for _ in range(5):
+        last = model.learn(x, t)
+    assert last < first
+    assert all(not torch.equal(a, b) for a, b in zip(before, model.msd.parameters()))
+
+
+def test_loss_gradient_scales_with_the_incoming_gradient():
+    # (3 * loss).backward() must give three times the gradients
+    from msd_pytorch_amd import MSDRegressionModel
+    torch.manual_seed(5)
+    model = MSDRegressionModel(1, 1, 4, 1)
+    model.msd.final_layer.linear.weight.data.normal_(0, 0.1)
+    x, t = torch.rand(1, 1, 32, 64), torch.rand(1, 1, 32, 64)
+    model._launch_forward(x, t)
+    model.optimizer.zero_grad()
+    model.loss.backward(retain_graph=True)
+    once = _grads(model)
+    model.optimizer.zero_grad()
+    (3 * model.loss).backward()
+    for name, g in _grads(model).items():
+        assert rel_err(g, 3 * once[name]) <= 1e-6, name
