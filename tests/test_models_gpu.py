@@ -480,6 +480,30 @@ def test_graphed_step_with_capturable_adam_follows_the_eager_optimiser():
     assert any(not torch.equal(p.detach(), b) for p, b in zip(captured.msd.parameters(), before))
 
 
+def test_train_with_a_recorded_step_follows_the_eager_loop():
+    # MSDModel.train(graph=True): the step of the first batch runs eagerly and is recorded, later
+    # batches replay it; the plain Adam of the model is switched to its capturable form with
+    # its state kept (one eager step was taken before)
+    from msd_pytorch_amd import MSDRegressionModel
+    size = (32, 64)
+    torch.manual_seed(21)
+    batches = [(torch.randn(1, 1, *size), torch.randn(1, 1, *size)) for _ in range(5)]
+    models = []
+    for _ in range(2):
+        torch.manual_seed(20)
+        m = MSDRegressionModel(1, 1, depth=5, width=1, dilations=[1, 2, 3])
+        m.msd.final_layer.linear.weight.data.normal_(0, 0.2)
+        m.learn(*batches[0])
+        models.append(m)
+    eager, recorded = models
+    eager.train(batches[1:], 2)
+    recorded.train(batches[1:], 2, graph=True)
+    assert recorded.optimizer.defaults["capturable"]
+    for a, b in zip(recorded.msd.parameters(), eager.msd.parameters()):
+        assert rel_err(a.detach(), b.detach()) <= 1e-5
+    assert abs(recorded.get_loss() - eager.get_loss()) <= 1e-5 * max(1.0, abs(eager.get_loss()))
+
+
 def test_regression_state_dict_keys():
     # key layout of the reference's checkpoints (msd_regression_model.py:76, msd_block.py:170-179)
     from msd_pytorch_amd import MSDRegressionModel
