@@ -634,7 +634,9 @@ template <int NDIM>
 int choose_vec(const Geom &g, int vmax, const View<const float> &gy, const View<const float> &x,
                const View<float> &gx, bool lng)
 {
-    for (int v = NDIM == 3 ? 2 : 4; v >= 1; v /= 2) {
+    // 3D: one voxel per lane only (27 gathered taps per voxel; the staged rows and the waves'
+    // tiles of two voxels per lane do not fit the LDS budget at any row length)
+    for (int v = NDIM == 3 ? 1 : 4; v >= 1; v /= 2) {
         if (v > vmax) continue;
         if (fits<NDIM>(g, v, gy, x, gx, lng)) return v;
     }
@@ -770,7 +772,9 @@ hipError_t xkb_nd(const Geom &g, const View<const float> &gy, const View<const f
         if (v == 4) return pick_ncb<2, 4, 1, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
     }
     if (g.Wd != 1) return hipErrorInvalidConfiguration;
-    if (v == 2) return pick_ncb<NDIM, 2, 1, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
+    if constexpr (NDIM == 2) {
+        if (v == 2) return pick_ncb<2, 2, 1, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
+    }
     if (v == 1) return pick_ncb<NDIM, 1, 1, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
     return hipErrorInvalidConfiguration;
 }

@@ -17,8 +17,9 @@ def bias_close(got, want, terms, tol=1e-4):
 
 
 def check_operator_problem(cc, shape, seed=7):
-    """conv_relu_forward, the three conv_relu_backward_* operators (accumulating) and the
-    three plain backward operators as one call (conv_backward_xkb), against the oracle."""
+    """conv_relu_forward and the three conv_relu_backward_* operators (accumulating), the plain
+    operators (conv_forward, conv_backward_x, conv_backward_kb) and the three plain backward
+    operators as one call (conv_backward_xkb), against the oracle."""
     ref = make_problem(shape, torch.float32, seed=seed)
     dev = make_problem(shape, torch.float32, device="cuda", seed=seed)
     d = ref["d"]
@@ -40,6 +41,23 @@ def check_operator_problem(cc, shape, seed=7):
     assert torch.equal(dev["gy"].cpu(), ref["gy"]), "conv_relu_backward_x wrote outside grad_input"
     assert rel_err(got_gk, want_gk) <= 1e-4, "conv_relu_backward_k"
     assert bias_close(got_gb, want_gb, ref["gy"] * (ref["y"] > 0)), "conv_relu_backward_bias"
+    # the plain (no-ReLU) operators one by one
+    ref3 = make_problem(shape, torch.float32, seed=seed + 2)
+    dev3 = make_problem(shape, torch.float32, device="cuda", seed=seed + 2)
+    want_gk, want_gb = torch.zeros_like(ref3["k"]), torch.zeros_like(ref3["bias"])
+    oracle.conv_forward(ref3["x"], ref3["k"], ref3["bias"], ref3["y"], d)
+    oracle.conv_backward_x(ref3["gy"], ref3["k"], ref3["gx"], d)
+    oracle.conv_backward_k(ref3["gy"], ref3["x"], want_gk, d)
+    oracle.conv_backward_bias(ref3["gy"], want_gb)
+    got_gk, got_gb = torch.zeros_like(dev3["k"]), torch.zeros_like(dev3["bias"])
+    cc.conv_forward(dev3["x"], dev3["k"], dev3["bias"], dev3["y"], d)
+    cc.conv_backward_x(dev3["gy"], dev3["k"], dev3["gx"], d)
+    cc.conv_backward_kb(dev3["gy"], dev3["x"], got_gk, got_gb, d)
+    torch.cuda.synchronize()
+    assert rel_err(dev3["stack"], ref3["stack"]) <= 1e-5, "conv_forward"
+    assert rel_err(dev3["gstack"], ref3["gstack"]) <= 1e-4, "conv_backward_x"
+    assert rel_err(got_gk, want_gk) <= 1e-4, "conv_backward_kb grad_kernel"
+    assert bias_close(got_gb, want_gb, ref3["gy"]), "conv_backward_kb grad_bias"
     # the three plain operators in one call
     ref2 = make_problem(shape, torch.float32, seed=seed + 1)
     dev2 = make_problem(shape, torch.float32, device="cuda", seed=seed + 1)

@@ -72,13 +72,60 @@ BACKWARD_X += [({"bwdx.vec3d": v, "bwdx.unroll3d": u}, s) for v in (1, 2, 4) for
 BACKWARD_X += [({"bwdx.min_blocks": n}, s) for n in (1, 4096) for s in (IMG_B, VOL_B)]
 
 
+# Template instances of the one-pass backward kernel that neither the cases above nor the
+# other test files reach: (voxels per lane, blocks of 16 channels per launch, output channels,
+# variant for unaligned or long rows) chosen by row length, channel count and width.
+INSTANCES = [
+    ({}, (1, 40, 1, (6, 1001), 3)),                  # odd rows: one voxel per lane, 33-64 channels
+    ({"bwdk.vec2d": 1}, (1, 70, 2, (8, 128), 2)),    # one voxel per lane, two output channels, > 64 channels
+    ({}, (1, 9, 2, (9, 256), 2)),                    # two voxels per lane, two output channels, one block
+    ({}, (1, 20, 1, (6, 750), 2)),                   # rows of whole pairs only: two voxels per lane, two blocks
+    ({}, (1, 20, 2, (9, 256), 3)),
+    ({"bwdk.vec2d": 2}, (1, 40, 1, (9, 256), 2)),
+    ({}, (1, 40, 1, (6, 750), 2)),
+    ({}, (1, 40, 2, (5, 1022), 4)),
+    ({"bwdk.vec2d": 2}, (1, 70, 1, (9, 256), 2)),
+    ({}, (1, 70, 2, (9, 256), 3)),
+    ({}, (1, 70, 2, (5, 1022), 4)),
+    ({}, (1, 40, 1, (5, 2048), 3)),                  # rows of two segments, 33-64 channels
+    ({}, (1, 70, 1, (5, 6, 64), 2)),                 # 3D, more than 64 channels
+    ({"bwdk.rows": 0, "bwdk.vec2d": 2}, (1, 40, 1, (9, 256), 2)),
+    ({"bwdk.rows": 0, "bwdk.vec2d": 2}, (1, 70, 1, (9, 256), 2)),
+    ({"bwdk.rows": 0, "bwdk.vec2d": 2}, (1, 3, 1, (9, 256), 2)),
+    ({"bwdk.rows": 0, "bwdk.vec2d": 4}, (1, 40, 1, (9, 256), 2)),
+    ({"bwdk.rows": 0, "bwdk.vec3d": 2}, (1, 40, 1, (5, 6, 128), 2)),
+    ({"bwdk.rows": 0, "bwdk.vec3d": 4}, (1, 3, 1, (5, 6, 128), 2)),
+    ({"bwdk.rows": 0, "bwdk.vec3d": 4}, (1, 20, 1, (5, 6, 128), 2)),
+    ({"bwdk.rows": 0, "bwdk.vec3d": 4}, (1, 40, 1, (5, 6, 128), 2)),
+    ({"bwdk.rows": 0, "bwdk.vec3d": 4}, (1, 70, 1, (5, 6, 128), 2)),
+    ({"bwdk.vec2d": 1}, (1, 40, 1, (9, 128), 2)),
+    ({"bwdk.vec2d": 2}, (1, 70, 1, (9, 128), 2)),
+    ({"bwdk.vec2d": 4}, (1, 70, 1, (9, 256), 2)),
+    ({"bwdk.vec3d": 1}, (1, 20, 1, (5, 6, 64), 2)),
+    ({"bwdk.vec3d": 1}, (1, 40, 1, (5, 6, 64), 2)),
+    ({"bwdk.vec3d": 2}, (1, 40, 1, (5, 6, 128), 2)),
+    ({"bwdk.vec3d": 2}, (1, 70, 1, (5, 6, 128), 2)),
+    ({"bwdx.vec2d": 4, "bwdx.unroll2d": 4}, (1, 5, 1, (4, 2048), 3)),     # rows of 512 lanes
+    ({"bwdx.vec2d": 4, "bwdx.unroll2d": 4}, (1, 5, 2, (4, 2048), 3)),
+    ({"bwdx.vec3d": 4, "bwdx.unroll3d": 2}, (1, 5, 1, (3, 4, 2048), 3)),
+    ({"bwdx.vec3d": 4, "bwdx.unroll3d": 4}, (1, 5, 2, (3, 4, 2048), 3)),
+    ({"bwdx.vec3d": 2, "bwdx.unroll3d": 2}, (1, 5, 1, (5, 6, 128), 2)),
+    ({"bwdx.vec3d": 1, "bwdx.unroll3d": 4}, (1, 5, 1, (5, 6, 128), 2)),
+    ({"fwd.vec3d": 2}, (1, 6, 1, (5, 6, 256), 2)),
+    ({"fwd.vec3d": 4}, (1, 6, 2, (5, 6, 256), 2)),
+    ({"fwd.vec3d": 2}, (1, 6, 2, (5, 6, 256), 2)),
+    ({"fwd.vec2d": 1}, (1, 6, 2, (9, 128), 2)),
+]
+
+
 def _id(case):
     settings, s = case
     knobs = ",".join("%s=%d" % kv for kv in settings.items())
     return "%s-B%d-C%d-w%d-%s-d%d" % (knobs, s[0], s[1], s[2], "x".join(map(str, s[3])), s[4])
 
 
-@pytest.mark.parametrize("case", FORWARD_2D + FORWARD_3D + SPLIT + ORDER + BACKWARD_K + BACKWARD_X, ids=_id)
+@pytest.mark.parametrize("case", FORWARD_2D + FORWARD_3D + SPLIT + ORDER + BACKWARD_K + BACKWARD_X + INSTANCES,
+                         ids=_id)
 def test_operators_under_a_forced_setting(cc, case):
     settings, shape = case
     with tuning(settings):
