@@ -6,7 +6,9 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libmsd_hip.so")
+# MSD_HIP_LIBRARY names another build of the library (same C ABI), e.g. one compiled with
+# different tuning constants, for side-by-side measurements
+LIB_PATH = os.environ.get("MSD_HIP_LIBRARY") or os.path.join(_HERE, "libmsd_hip.so")
 ABI_VERSION = 1
 
 MSD_F32, MSD_F64 = 0, 1

@@ -118,8 +118,9 @@ hipError_t launch(const Geom &g, const View<const float> &out, const View<const 
     if (rt.lpr * rt.rpw <= 256) {
         hipLaunchKernelGGL((bwdx_rows<NDIM, RELU, WOUT, V, U, 256>), grid, dim3(rt.lpr * rt.rpw), lds,
                            s, g, rt, cch, remap, out, gy, k, gx, pm);
-    } else if constexpr (V == 4) {
-        // rows longer than 1024 voxels: up to 1024 lanes per workgroup
+    } else if constexpr (V == 4 && !(NDIM == 3 && WOUT == 2)) {
+        // rows longer than 1024 voxels: up to 1024 lanes per workgroup (3D with two output
+        // channels: the 18 staged rows of such a row do not fit the LDS budget, see fits())
         hipLaunchKernelGGL((bwdx_rows<NDIM, RELU, WOUT, V, U, 1024>), grid, dim3(rt.lpr * rt.rpw), lds,
                            s, g, rt, cch, remap, out, gy, k, gx, pm);
     } else {

@@ -78,8 +78,9 @@ struct Args {
 // Workgroups (of four waves) that are resident per CU: the 3D kernel with one voxel per lane
 // and at most 64 channels per chunk fits 168 registers (with pipeline stages of 16 voxels),
 // so three of them share a CU; the others need up to 256 registers, which leaves room for
-// two.  (Four per CU are slower, by 2 % at 16 channels even where the 128 registers they
-// leave cost only six spilled registers: three is where the gain ends.)
+// two.  (Four per CU are slower, by 10 %: the 128 registers they leave cost 15 to 22 spilled
+// registers, also with the gather's LDS reads held a third at a time: three is where the
+// gain ends.)
 template <int NDIM, int V, int NCB, int WOUT> constexpr int resident_per_cu()
 {
     return (NDIM == 3 && V == 1 && WOUT == 1 && NCB <= 4) ? 3 : 2;

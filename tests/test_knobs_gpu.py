@@ -115,6 +115,13 @@ INSTANCES = [
     ({"fwd.vec3d": 4}, (1, 6, 2, (5, 6, 256), 2)),
     ({"fwd.vec3d": 2}, (1, 6, 2, (5, 6, 256), 2)),
     ({"fwd.vec2d": 1}, (1, 6, 2, (9, 128), 2)),
+    ({"bwdk.vec2d": 2}, (1, 9, 2, (9, 256), 2)),
+    ({"bwdk.vec2d": 2}, (1, 70, 2, (9, 256), 3)),
+    ({"bwdk.vec2d": 1}, (1, 20, 1, (9, 128), 2)),
+    ({"bwdx.vec2d": 1, "bwdx.unroll2d": 4}, (1, 6, 2, (9, 128), 2)),
+    ({"bwdx.vec3d": 4, "bwdx.unroll3d": 2}, (1, 5, 1, (3, 4, 1536), 3)),   # 3D rows of 384 lanes
+    ({"bwdx.vec3d": 4, "bwdx.unroll3d": 4}, (1, 5, 1, (3, 4, 1536), 3)),
+    ({"bwdx.vec3d": 4, "bwdx.unroll3d": 4}, (1, 5, 2, (3, 4, 768), 3)),
 ]
 
 

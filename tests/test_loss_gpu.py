@@ -37,6 +37,11 @@ CASES = [
     (2, 5, 4, (6, 10, 12)),
     (1, 21, 5, (40, 44)),
     (2, 3, 8, (5, 6, 8)),
+    # odd plane sizes with 1, 4 and 8 output channels; an even one with 2
+    (1, 4, 1, (7, 9)),
+    (2, 6, 4, (3, 5, 7)),
+    (1, 5, 8, (9, 11)),
+    (1, 9, 2, (8, 12)),
 ]
 
 

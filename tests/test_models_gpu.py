@@ -545,6 +545,10 @@ def test_segmentation_model_api(ndim, tmp_path):
     ((1, 9, 8, 40), 11, torch.float32),        # more output channels than one launch takes (8 + 2 + 1)
     ((2, 6, 9, 10), 2, torch.float64),
     ((1, 3, 4, 6, 10), 5, torch.float64),
+    # odd voxel counts (one voxel per thread) with every group width of output channels, both types
+    ((1, 6, 7, 9), 13, torch.float32),         # 8 + 4 + 1
+    ((1, 5, 3, 5, 7), 15, torch.float64),      # 8 + 4 + 2 + 1
+    ((2, 4, 6, 10), 8, torch.float64),         # two voxels per thread, 8 output channels
 ])
 def test_final_layer_matches_conv1d(shape, c_out, dtype):
     # the native final layer against the Conv1d over flattened voxels it replaces
