@@ -75,15 +75,15 @@ struct Args {
     RowSegments sg;      // LONG instances
 };
 
-// Workgroups (of four waves) that are resident per CU: the 3D kernel with one voxel per lane
-// and at most 64 channels per chunk fits 168 registers (with pipeline stages of 16 voxels),
-// so three of them share a CU; the others need up to 256 registers, which leaves room for
-// two.  (Four per CU are slower, by 10 %: the 128 registers they leave cost 15 to 22 spilled
-// registers, also with the gather's LDS reads held a third at a time: three is where the
-// gain ends.)
+// Workgroups (of four waves) that are resident per CU.  The 3D kernel with one voxel per lane
+// (pipeline stages of 16 voxels, arguments read again per tile, see the tile loop) needs 107 and
+// 115 registers with up to 16 and 32 channels per chunk: four workgroups share a CU (8.70 ->
+// 8.54 ms for the backward pass of a 50-layer network at 128^3).  With up to 64 channels per
+// chunk it needs 131, three per CU (forced into the 128 registers of four it spills 15 of them
+// and is slower).  The others need up to 256 registers, which leaves room for two.
 template <int NDIM, int V, int NCB, int WOUT> constexpr int resident_per_cu()
 {
-    return (NDIM == 3 && V == 1 && WOUT == 1 && NCB <= 4) ? 3 : 2;
+    return (NDIM == 3 && V == 1 && WOUT == 1 && NCB <= 4) ? (NCB <= 2 ? 4 : 3) : 2;
 }
 
 // Register sets of the channel loop's load pipeline: the loads of stage s + NSETS - 1 are
@@ -105,7 +105,7 @@ template <int NDIM, int V, int NCB, int WOUT, bool LONG> constexpr int pipeline_
 // instance because even its few extra scalar instructions per stage cost the plain one 1-4 %.
 template <int NDIM, int V, int NCB, int WOUT, bool LONG>
 __global__ __launch_bounds__(kThreads, (resident_per_cu<NDIM, V, NCB, WOUT>()))
-void bwd_rows_fused(const Args a, const float *__restrict__ gyp, const float *__restrict__ xp,
+void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *__restrict__ xp,
                     float *__restrict__ gxp, const float *__restrict__ actp, const float *__restrict__ kw,
                     float *__restrict__ part)
 {
@@ -132,6 +132,7 @@ void bwd_rows_fused(const Args a, const float *__restrict__ gyp, const float *__
     static_assert(!XPAIR || (H == 4 && NSETS == 2), "a block is two pairs of stages");
     static_assert(H % NSETS == 0 && NSETS >= 2, "the stages of a block rotate through the register sets");
     constexpr int ASTRIDE = ATile<NDIM, V, WOUT>::kStride;
+    const Args &a = a_;
     const Geom &g = a.g;
     const RowTeams &rt = a.rt;
     const int tid = threadIdx.x;
@@ -186,7 +187,26 @@ void bwd_rows_fused(const Args a, const float *__restrict__ gyp, const float *__
     int row = gi * rt.rpw + team;
     int y = row % g.H, z = row / g.H;
 
-    for (int ti = 0; ti < a.tiles_per_wg; ti++) {
+    // The kernel's arguments are the first thing in the argument block.  The 3D instances read
+    // them again from there for every tile (scalar loads) instead of keeping them over the
+    // channel loop, which has the scalar registers full of weights: kept, they are spilled to
+    // lanes of a vector register, every use costs a vector instruction, and the register
+    // allocation around them grows (3D, up to 32 channels per chunk: 142-150 -> 108-116 VGPRs,
+    // which is what lets a fourth workgroup share the CU).  2D is 2 % slower that way.
+    constexpr bool RELOAD = NDIM == 3;
+    typedef const __attribute__((address_space(4))) int *kernarg_words_t;
+    kernarg_words_t kernarg = (kernarg_words_t)__builtin_amdgcn_kernarg_segment_ptr();
+    for (int ti = 0; ti < a_.tiles_per_wg; ti++) {
+        Args a = a_;
+        if constexpr (RELOAD) {
+            static_assert(sizeof(Args) % sizeof(int) == 0, "Args is made of ints");
+            asm volatile("" : "+s"(kernarg));     // a new address as far as the compiler knows: loaded again
+            int *dst = reinterpret_cast<int *>(&a);
+#pragma unroll
+            for (int i = 0; i < (int)(sizeof(Args) / sizeof(int)); i++) dst[i] = kernarg[i];
+        }
+        const Geom &g = a.g;
+        const RowTeams &rt = a.rt;
         if (grp >= a.total_groups) break;         // uniform over the workgroup
         int xsc = a.x.sc, gsc = a.gx.sc;
         asm volatile("" : "+s"(xsc), "+s"(gsc));  // keeps per-channel addresses from being hoisted out of the loop
