@@ -197,14 +197,17 @@ void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *_
     typedef const __attribute__((address_space(4))) int *kernarg_words_t;
     kernarg_words_t kernarg = (kernarg_words_t)__builtin_amdgcn_kernarg_segment_ptr();
     for (int ti = 0; ti < a_.tiles_per_wg; ti++) {
-        Args a = a_;
+        Args again;
         if constexpr (RELOAD) {
             static_assert(sizeof(Args) % sizeof(int) == 0, "Args is made of ints");
             asm volatile("" : "+s"(kernarg));     // a new address as far as the compiler knows: loaded again
-            int *dst = reinterpret_cast<int *>(&a);
+            int *dst = reinterpret_cast<int *>(&again);
 #pragma unroll
             for (int i = 0; i < (int)(sizeof(Args) / sizeof(int)); i++) dst[i] = kernarg[i];
         }
+        const Args &a = [&]() -> const Args & {
+            if constexpr (RELOAD) return again; else return a_;
+        }();
         const Geom &g = a.g;
         const RowTeams &rt = a.rt;
         if (grp >= a.total_groups) break;         // uniform over the workgroup
@@ -227,8 +230,14 @@ void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *_
         const uint64_t abase = reinterpret_cast<uint64_t>(actp + (int64_t)b * a.gx.sb);
         uint32_t goff = 4u * (uint32_t)(zc * a.gx.sz + yc * a.gx.sy + xc);
         // uniform base of grad_input channel ci, kept in scalar registers
+        // (plain instances: the whole of grad_input is below 2^30 values, xkb_mode(), so the
+        // channel's byte offset is a 32-bit product: three scalar instructions instead of seven)
         auto channel_base = [&](uint64_t base, int ci) {
-            uint64_t p = base + (uint64_t)((int64_t)ci * gsc * 4);
+            uint64_t p;
+            if constexpr (LONG)
+                p = base + (uint64_t)((int64_t)ci * gsc * 4);
+            else
+                p = base + (uint64_t)((uint32_t)ci * (uint32_t)gsc * 4u);
             asm volatile("" : "+s"(p));
             return p;
         };
@@ -389,7 +398,7 @@ void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *_
         auto load_weights = [&](int ci, float (&w)[KR]) {
 #pragma unroll
             for (int co = 0; co < WOUT; co++) {
-                const float *kc = kw + ((int64_t)co * g.C + ci) * K;
+                const float *kc = kw + (uint32_t)((co * g.C + ci) * K);
 #pragma unroll
                 for (int t = 0; t < K; t++) w[co * K + t] = kc[t];
             }
@@ -734,7 +743,8 @@ hipError_t pick_ncb(const Geom &g, const View<const float> &gy, const View<const
 constexpr int kMaxVecTwoOutputs = 2;
 
 // Lane offsets into x fit 32 bits: they span the whole stack in the plain kernel, one block
-// of 16 channels in the LONG one.
+// of 16 channels in the LONG one.  The plain kernel asks the same of grad_input (its channel
+// offsets are 32-bit products).
 inline bool x_offsets_fit(const Geom &g, const View<const float> &x, bool lng)
 {
     const int64_t channels = lng ? kChanBlock : g.C;
@@ -752,7 +762,9 @@ Mode xkb_mode(const Geom &g, const View<const float> &gy, const View<const float
     if (x.sx != 1 || gy.sx != 1 || gx.sx != 1) return kUnsupported;
     if (!small_strides(g, gy) || !small_strides(g, x) || !small_strides(g, gx)) return kUnsupported;
     const int vmax = g.Wd == 2 ? kMaxVecTwoOutputs : 4;
-    if (x_offsets_fit(g, x, false) && choose_vec<NDIM>(g, vmax, gy, x, gx, false) != 0) return kPlain;
+    const View<const float> gxc{gx.p, gx.sb, gx.sc, gx.sz, gx.sy, gx.sx};
+    if (x_offsets_fit(g, x, false) && x_offsets_fit(g, gxc, false) && choose_vec<NDIM>(g, vmax, gy, x, gx, false) != 0)
+        return kPlain;
     if (x_offsets_fit(g, x, true) && choose_vec<NDIM>(g, vmax, gy, x, gx, true) != 0) return kLong;
     return kUnsupported;
 }
