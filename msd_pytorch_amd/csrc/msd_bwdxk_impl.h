@@ -76,14 +76,13 @@ struct Args {
 };
 
 // Workgroups (of four waves) that are resident per CU.  The 3D kernel with one voxel per lane
-// (pipeline stages of 16 voxels, arguments read again per tile, see the tile loop) needs 107 and
-// 115 registers with up to 16 and 32 channels per chunk: four workgroups share a CU (8.70 ->
-// 8.54 ms for the backward pass of a 50-layer network at 128^3).  With up to 64 channels per
-// chunk it needs 131, three per CU (forced into the 128 registers of four it spills 15 of them
-// and is slower).  The others need up to 256 registers, which leaves room for two.
-template <int NDIM, int V, int NCB, int WOUT> constexpr int resident_per_cu()
+// (pipeline stages of 16 voxels, arguments read again per tile, row arithmetic on the scalar
+// pipe, see the tile loop) needs 94 to 118 registers with up to 64 channels per chunk: four
+// workgroups share a CU; with up to 128 channels it needs 167, three per CU (the LONG variant of
+// that one would spill: two).  The others need up to 256 registers, which leaves room for two.
+template <int NDIM, int V, int NCB, int WOUT, bool LONG> constexpr int resident_per_cu()
 {
-    return (NDIM == 3 && V == 1 && WOUT == 1 && NCB <= 4) ? (NCB <= 2 ? 4 : 3) : 2;
+    return (NDIM == 3 && V == 1 && WOUT == 1) ? (NCB <= 4 ? 4 : (LONG ? 2 : 3)) : 2;
 }
 
 // Register sets of the channel loop's load pipeline: the loads of stage s + NSETS - 1 are
@@ -104,7 +103,7 @@ template <int NDIM, int V, int NCB, int WOUT, bool LONG> constexpr int pipeline_
 // `dil` values on either side.  It is a separate
 // instance because even its few extra scalar instructions per stage cost the plain one 1-4 %.
 template <int NDIM, int V, int NCB, int WOUT, bool LONG>
-__global__ __launch_bounds__(kThreads, (resident_per_cu<NDIM, V, NCB, WOUT>()))
+__global__ __launch_bounds__(kThreads, (resident_per_cu<NDIM, V, NCB, WOUT, LONG>()))
 void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *__restrict__ xp,
                     float *__restrict__ gxp, const float *__restrict__ actp, const float *__restrict__ kw,
                     float *__restrict__ part)
@@ -139,7 +138,12 @@ void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *_
     const int nwaves = blockDim.x / kWave;
     const int wave = __builtin_amdgcn_readfirstlane(tid / kWave), wl = tid % kWave;
     const int mk = wl / 16, mj = wl % 16;         // MFMA k (voxel group) and i/j (tap or channel) of this lane
-    const int team = tid / rt.lpr, lane = tid % rt.lpr;
+    // a row team is whole waves (fits()), so the team and everything derived from its row
+    // (the source rows of the gather, their clamps and addresses) is wave-uniform: computed
+    // from the wave number, it stays in scalar registers and on the scalar pipe
+    // (2D keeps the per-lane form: there the scalar registers are the scarcer ones)
+    const int team = NDIM == 3 ? (wave * kWave) / rt.lpr : tid / rt.lpr;
+    const int lane = tid - team * rt.lpr;
     // segments (rt.segs > 1): a tile is one segment of one row
     constexpr bool SEG = LONG;
     const bool segmented = SEG && a.sg.segs > 1;  // uniform
@@ -690,7 +694,7 @@ hipError_t launch(const Geom &g, const View<const float> &gy, const View<const f
     a.remap = knob(kKnobXcdRemap, 1);
     // as many workgroups as are resident at once (256 CUs): the grid then runs as one round
     const int64_t max_wgs = std::min<int64_t>(
-        std::max(8, knob(kKnobBwdkBlocks, 256 * resident_per_cu<NDIM, V, NCB, WOUT>())), kMaxPartialRows);
+        std::max(8, knob(kKnobBwdkBlocks, 256 * resident_per_cu<NDIM, V, NCB, WOUT, LONG>())), kMaxPartialRows);
     a.tiles_per_wg = (int)((total + max_wgs - 1) / max_wgs);
     const int64_t wgs = (total + a.tiles_per_wg - 1) / a.tiles_per_wg;
     const int rows = a.remap ? xcd_grid((int)wgs) : (int)wgs;   // padding workgroups write zero rows
