@@ -169,7 +169,7 @@ def kernel_times(lib, torch, run_steps):
     return {n: (ms[i], calls[i]) for i, n in enumerate(names)}
 
 
-def cpu_baseline(name, budget_s=12.0):
+def cpu_baseline(name, budget_s=15.0):
     """Time the CPU oracle's dense-block forward+backward on a bounded sample:
     the same network on a smaller image, sized from a calibration run."""
     import torch
