@@ -115,7 +115,7 @@ def make_model(name, torch):
     return model
 
 
-def algorithmic_work(name, fused):
+def algorithmic_work(name, fused, paired=False):
     """Per-step algorithmic bytes and flops of each kernel class, fp32, per layer with C input
     and w output channels over N voxels and K = 9 or 27 taps:
     bytes: forward (C + w) N 4, backward_x (2C + 2w) N 4, backward_k+bias (C + 2w) N 4, the fused
@@ -124,14 +124,30 @@ def algorithmic_work(name, fused):
     flops: 2 C w K N for each of forward, backward_x and backward_k (the fused pass does two).
     `fused` says which way the library ran the layers above the first (it reports a
     non-zero call count for the fused class); layer 0 needs no input gradient.
+    `paired`: the library runs the layers of a 2D block of width 1 two at a time (layers i and
+    i - 1, from the top, while i - 1 > 0): one fused pass over layer i's last input channel
+    alone, (3 + 2) N 4 bytes, and one over the c channels below both layers with the two layers
+    as its two output channels, (3c + 4) N 4 bytes: what that algorithm has to move, which is
+    about half of the per-layer figure.  The per-layer figure is returned as well, under
+    "backward_xkb_per_layer".
     Returns (bytes per class, flops per class, voxels per step)."""
     kind, ndim, c_in, c_out, depth, width, batch, spatial, adam = WORKLOADS[name]
     n = batch
     for s in spatial:
         n *= s
     K = 3 ** ndim
-    nbytes = {"forward": 0, "backward_x": 3 * width * n * 4, "backward_kb": 0, "backward_xkb": 0}
+    nbytes = {"forward": 0, "backward_x": 3 * width * n * 4, "backward_kb": 0, "backward_xkb": 0,
+              "backward_xkb_per_layer": 0}
     flops = {"forward": 0, "backward_x": 0, "backward_kb": 0, "backward_xkb": 0}
+    in_pair = set()
+    if fused and paired:
+        i = depth - 1
+        while i - 1 > 0:
+            in_pair.update((i, i - 1))
+            c = c_in + width * (i - 1)           # channels below both layers
+            nbytes["backward_xkb"] += (3 + 2) * n * 4 + 2 * K * 4
+            nbytes["backward_xkb"] += (3 * c + 4) * n * 4 + 2 * (2 * c * K * 4)
+            i -= 2
     for i in range(depth):
         C = c_in + width * i
         wts = width * C * K * 4
@@ -139,7 +155,10 @@ def algorithmic_work(name, fused):
         nbytes["forward"] += (C + width) * n * 4 + wts
         flops["forward"] += op
         if i > 0 and fused:
-            nbytes["backward_xkb"] += (3 * C + 2 * width) * n * 4 + 2 * wts
+            per_layer = (3 * C + 2 * width) * n * 4 + 2 * wts
+            nbytes["backward_xkb_per_layer"] += per_layer
+            if i not in in_pair:
+                nbytes["backward_xkb"] += per_layer
             flops["backward_xkb"] += 2 * op
             continue
         if i > 0:
@@ -250,7 +269,10 @@ def measure(name, args, lib, torch):
 
     if not args.no_kernel_timing:
         totals = kernel_times(lib, torch, lambda: [eager_step() for _ in range(args.steps)])
-        bytes_per_step, flops_per_step, _ = algorithmic_work(name, totals["backward_xkb"][1] > 0)
+        # 2D blocks of width 1 run their layers two at a time in the backward pass (block.pair)
+        paired = ndim == 2 and width == 1 and not any(kv.replace(" ", "") in ("block.pair=0", "block.fuse=0")
+                                                      for kv in args.tune)
+        bytes_per_step, flops_per_step, _ = algorithmic_work(name, totals["backward_xkb"][1] > 0, paired)
         kernels = {}
         for cls, (ms, launches) in totals.items():
             if launches == 0:
@@ -265,6 +287,12 @@ def measure(name, args, lib, torch):
                             "algorithmic_GFLOP_per_step": round(flops_per_step[cls] / 1e9, 2),
                             "TFLOPs": round(tfl, 2), "frac_fp32": round(tfl / FP32_PEAK_TFLOPS, 4),
                             "Mvoxel_per_s": round(nvox / per_step_s / 1e6, 2)}
+            if cls == "backward_xkb" and paired:
+                # the same time priced with the bytes of one fused pass per layer, for comparison
+                per_layer = bytes_per_step["backward_xkb_per_layer"]
+                kernels[cls]["layers_in_pairs"] = True
+                kernels[cls]["per_layer_GB_per_step"] = round(per_layer / 1e9, 3)
+                kernels[cls]["per_layer_GBps"] = round(per_layer / per_step_s / 1e9, 1)
         dominant = max(kernels, key=lambda c: kernels[c]["ms_per_step"])
         dom = kernels[dominant]
         # the committed counter figures describe the library's default launch shapes

@@ -77,7 +77,8 @@ int msd_set_kernel_path(int path);
  * "block.defer" (0/1: one reduction launch for many layers), "block.snake" (0/1: alternate
  * layers walk the channels in opposite directions), "fwd.class3d" (0/1: 3D forward tiles
  * numbered by residue class), "fwd.lattice3d" (24, 33 or 44: rows z x y of a 3D forward tile;
- * 0: chosen by the library).  Unknown keys return MSD_ERR_INVALID.
+ * 0: chosen by the library), "block.pair" (0/1: the backward pass of a 2D block of one-channel
+ * layers takes its layers two at a time).  Unknown keys return MSD_ERR_INVALID.
  */
 int msd_set_tuning(const char *key, int value);
 

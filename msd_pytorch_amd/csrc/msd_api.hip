@@ -17,8 +17,9 @@ const char *const kKnobNames[kKnobCount] = {
     "xcd_remap", "bwdk.vec2d", "bwdk.vec3d", "bwdk.blocks",
     "fwd.vec2d", "fwd.vec3d", "fwd.split", "fwd.rows2d", "bwdk.rows", "block.fuse",
     "block.defer", "bwdk.interleave", "block.snake", "fwd.class3d", "fwd.lattice3d",
+    "block.pair",
 };
-static_assert(kKnobFwdLattice3d + 1 == kKnobCount, "one name per knob, in the order of the enum");
+static_assert(kKnobBlockPair + 1 == kKnobCount, "one name per knob, in the order of the enum");
 int g_knobs[kKnobCount];
 // every knob starts at "library default"
 const bool g_knobs_ready = [] {
@@ -718,8 +719,13 @@ int64_t block_layer_workspace(int dtype, int ndim, int64_t batch, int64_t c_in, 
     int64_t total = c_in, need = 0;
     for (int i = 0; i < depth; i++) {
         if (widths[i] <= 0) return -1;
-        const int64_t n = msd_workspace_bytes(dtype, ndim, batch, total, widths[i], spatial);
+        int64_t n = msd_workspace_bytes(dtype, ndim, batch, total, widths[i], spatial);
         if (n < 0) return -1;
+        if (i + 1 < depth && ndim == 2 && widths[i] == 1 && widths[i + 1] == 1) {
+            // this layer and the one above it may run as the two output channels of one pass
+            const int64_t n2 = msd_workspace_bytes(dtype, ndim, batch, total, 2, spatial);
+            n = n2 > n ? n2 : n;
+        }
         need = n > need ? n : need;
         total += widths[i];
     }
@@ -804,6 +810,91 @@ int block_layer_fused(const char *fn, const BlockArgs &a, int i, int64_t first, 
     return MSD_OK;
 }
 
+// Two layers of the block backward pass, i and i - 1 (2D, one output channel each), in two
+// launches instead of two full passes.  Layer i's inputs are the channels [0, first), layer
+// i - 1's the channels [0, first - 1); channel c = first - 1 is layer i - 1's output.
+//   1. layer i alone on channel c: its grad_input contribution completes that channel's
+//      gradient (masked with the channel's activation on the way out: it is layer i - 1's
+//      output gradient from here on), plus the nine weight gradients of that channel;
+//   2. both layers on the channels [0, c) as the two output channels of ONE pass of the fused
+//      kernel (each with its own dilation and weights): every channel of the input and of
+//      grad_input is moved once for the two layers, and both bias gradients are formed there.
+// *done is false (and nothing was launched) when the case is not covered.
+bool pair_candidate(const BlockArgs &a, int i, bool need_input_grad)
+{
+    return a.dtype == MSD_F32 && a.ndim == 2 && g_kernel_path == 0 && i >= 1 && a.widths[i] == 1 &&
+           a.widths[i - 1] == 1 && (i - 1 > 0 || need_input_grad) && msd::knob(msd::kKnobBlockFuse, 1) &&
+           msd::knob(msd::kKnobBlockPair, 1);
+}
+
+int block_pair_fused(const char *fn, const BlockArgs &a, int i, int64_t first, const void *stack,
+                     const int64_t *stack_strides, void *grads, const int64_t *grads_strides,
+                     const void *const *weights, void *const *grad_weights, void *gb_lower, void *ws, int64_t ws_bytes,
+                     hipStream_t s, DeferredReductions *pending, bool *masked, bool *done)
+{
+    *done = false;
+    if (!grad_weights[i] || !grad_weights[i - 1] || !gb_lower) return MSD_OK;
+    const int64_t c = first - 1;                  // channels below both layers; index of layer i - 1's output
+    const int d_hi = (int)a.dilations[i], d_lo = (int)a.dilations[i - 1];
+    constexpr int K = 9;
+    msd::Geom g1, g2;
+    MSD_TRY(make_geom(fn, a.dtype, a.ndim, a.batch, 1, 1, a.spatial, d_hi, true, &g1));
+    MSD_TRY(make_geom(fn, a.dtype, a.ndim, a.batch, c, 2, a.spatial, d_hi > d_lo ? d_hi : d_lo, true, &g2));
+    msd::View<const float> x, x1, gy1, gy2;
+    msd::View<float> gx, gx1;
+    MSD_TRY(make_view(fn, "input", a.ndim, stack, stack_strides, &x));
+    MSD_TRY(make_view(fn, "grad_input", a.ndim, grads, grads_strides, &gx));
+    // the activations are read through grad_input's addressing: same strides and alignment
+    const bool same_layout = x.sb == gx.sb && x.sc == gx.sc && x.sz == gx.sz && x.sy == gx.sy &&
+                             reinterpret_cast<uintptr_t>(x.p) % 16 == reinterpret_cast<uintptr_t>(gx.p) % 16;
+    if (!same_layout) return MSD_OK;
+    x1 = x;
+    x1.p += c * x.sc;
+    gx1 = gx;
+    gx1.p += c * gx.sc;
+    gy1 = msd::View<const float>{gx.p + first * gx.sc, gx.sb, gx.sc, gx.sz, gx.sy, gx.sx};   // layer i's output gradient
+    gy2 = msd::View<const float>{gx.p + c * gx.sc, gx.sb, gx.sc, gx.sz, gx.sy, gx.sx};       // layer i - 1's, then layer i's
+    if (!msd::fast_backward_xkb_supported(g1, gy1, x1, gx1) || !msd::fast_backward_xkb_supported(g2, gy2, x, gx))
+        return MSD_OK;
+    MSD_TRY(check_workspace(fn, g1, sizeof(float), ws, ws_bytes));
+    MSD_TRY(check_workspace(fn, g2, sizeof(float), ws, ws_bytes));
+    const float *w_hi = (const float *)weights[i], *w_lo = (const float *)weights[i - 1];
+    float *gk_hi = (float *)grad_weights[i], *gk_lo = (float *)grad_weights[i - 1];
+    {
+        // 1. channel c, layer i; the channel is an output of the layer below: masked on the way out
+        const msd::PostMask pm{0, x1};
+        const int64_t region = partial_region_floats(a.ndim, 1, 1);
+        msd::ReduceJob *job = nullptr;
+        MSD_TRY(pending->next(fn, region, &job));
+        ProfileScope scope(3, s);
+        const hipError_t e = msd::fast_backward_xkb(g1, gy1, x1, w_hi + c * K, gx1, pm, gk_hi + c * K, nullptr,
+                                                    (float *)ws, s, job);
+        if (e != hipSuccess) return hip_fail(fn, e);
+        if (job) pending->taken(region);
+    }
+    {
+        // 2. channels [0, c), both layers; the outputs of layer i - 2 are complete with this update
+        msd::PostMask pm{g2.C, {nullptr, 0, 0, 0, 0, 0}};
+        *masked = false;
+        if (i - 2 >= 0) {
+            pm = msd::PostMask{(int)(c - a.widths[i - 2]), x};
+            *masked = true;
+        }
+        const int64_t region = partial_region_floats(a.ndim, c, 2);
+        msd::ReduceJob *job = nullptr;
+        MSD_TRY(pending->next(fn, region, &job));
+        ProfileScope scope(3, s);
+        g2.reverse = msd::knob(msd::kKnobBlockSnake, 1) && ((i >> 1) & 1);
+        const msd::LayerPair pair{d_lo, d_hi, w_hi, gk_hi};
+        const hipError_t e = msd::fast_backward_xkb_2d(g2, gy2, x, w_lo, gx, pm, gk_lo, (float *)gb_lower, (float *)ws, s,
+                                                       job, &pair);
+        if (e != hipSuccess) return hip_fail(fn, e);
+        if (job) pending->taken(region);
+    }
+    *done = true;
+    return MSD_OK;
+}
+
 }  // namespace
 
 int64_t msd_block_workspace_bytes(int dtype, int ndim, int64_t batch, int64_t c_in, int depth, const int64_t *widths,
@@ -816,8 +907,9 @@ int64_t msd_block_workspace_bytes(int dtype, int ndim, int64_t batch, int64_t c_
     // their reductions can wait for one another
     int64_t regions = 0, total = c_in;
     for (int i = 0; i < depth; i++) {
-        if (dtype == MSD_F32 && widths[i] <= 2)
-            regions += partial_region_floats(ndim, total, widths[i]) * (int64_t)sizeof(float);
+        if (dtype == MSD_F32 && widths[i] <= 2)   // (+ the extra columns of a layer pair's first step)
+            regions += (partial_region_floats(ndim, total, widths[i]) + 16 * (int64_t)msd::kMaxPartialRows) *
+                       (int64_t)sizeof(float);
         total += widths[i];
     }
     return need + (regions < kDeferBudgetBytes ? regions : kDeferBudgetBytes);
@@ -884,6 +976,19 @@ int msd_block_backward(int dtype, int ndim, int64_t batch, int64_t c_in, int dep
                                            grads_strides, stream));
         masked = false;
         void *gb = grad_bias ? (char *)grad_bias + b0 * a.elem : nullptr;
+        if (pair_candidate(a, i, need_input_grad != 0)) {
+            // this layer and the one below it in two launches that move every shared channel once
+            bool done = false;
+            MSD_TRY(block_pair_fused(fn, a, i, first, stack, stack_strides, grads, grads_strides, weights, grad_weights,
+                                     grad_bias ? (char *)grad_bias + (b0 - 1) * a.elem : nullptr, workspace,
+                                     workspace_bytes, (hipStream_t)stream, &pending, &masked, &done));
+            if (done) {
+                last = first - 1;
+                b1 = b0 - 1;
+                i--;
+                continue;
+            }
+        }
         if (i > 0 || need_input_grad) {
             // one pass for the input, weight and bias gradients where the fused kernel applies
             bool done = false;

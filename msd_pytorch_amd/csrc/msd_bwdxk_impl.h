@@ -73,6 +73,7 @@ struct Args {
     int mask_from;       // activations (viewed like grad_input) mask the channels >= mask_from
     int want_bias;
     RowSegments sg;      // LONG instances
+    int dil1;            // two output channels: the dilation of the second one's taps (two layers in one pass)
 };
 
 // Workgroups (of four waves) that are resident per CU.  The 3D kernel with one voxel per lane
@@ -106,7 +107,7 @@ template <int NDIM, int V, int NCB, int WOUT, bool LONG>
 __global__ __launch_bounds__(kThreads, (resident_per_cu<NDIM, V, NCB, WOUT, LONG>()))
 void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *__restrict__ xp,
                     float *__restrict__ gxp, const float *__restrict__ actp, const float *__restrict__ kw,
-                    float *__restrict__ part)
+                    const float *__restrict__ kw1, float *__restrict__ part)
 {
     // the pointers are separate arguments so that they can carry __restrict__: the weights
     // are then known not to change under the stores to grad_input and stay scalar loads
@@ -310,37 +311,39 @@ void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *_
             const View<const float> gyv{gyp, a.gy.sb, a.gy.sc, a.gy.sz, a.gy.sy, 1};
             float own[WOUT][NPQ][V];
             if (segmented) {
-                if constexpr (SEG) stage_source_segment<NDIM, WOUT, V>(g, rt, a.sg, gyv, b, zc, yc, xs, lane, rowok, S, own);
+                if constexpr (SEG)
+                    stage_source_segment<NDIM, WOUT, V>(g, rt, a.sg, gyv, b, zc, yc, xs, lane, rowok, S, own, a.dil1);
             } else {
-                stage_source_rows<NDIM, false, WOUT, V>(g, rt, none, gyv, b, zc, yc, lane, act, S, own);
+                stage_source_rows<NDIM, false, WOUT, V>(g, rt, none, gyv, b, zc, yc, lane, act, S, own, a.dil1);
             }
             // per voxel: all LDS reads first, so that their latencies overlap, then the sums
 #pragma unroll
-            for (int i = 0; i < V; i++) {
-                const SideTaps<V> side = segmented
-                                             ? SideTaps<V>(x0 + i, g.W, g.dil, rt.lpr, xs, V * rt.lpr)
-                                             : SideTaps<V>(min(x0 + i, g.W - 1), g.W, g.dil, rt.lpr);
-                float ra[WOUT * NPQ][4];
+            for (int i = 0; i < V; i++)
 #pragma unroll
-                for (int pq = 0; pq < WOUT * NPQ; pq++) {
-                    const float *srow = S + (size_t)pq * rs;
-                    ra[pq][0] = srow[side.i0a];
-                    ra[pq][1] = srow[side.i0b];
-                    ra[pq][2] = srow[side.i2a];
-                    ra[pq][3] = srow[side.i2b];
-                }
-                __builtin_amdgcn_sched_barrier(0);
+                for (int co = 0; co < WOUT; co++) {
+                    // (the second output channel may have a dilation of its own, and with it its own x-taps)
+                    const int dil = (WOUT > 1 && co > 0 && a.dil1 > 0) ? a.dil1 : g.dil;
+                    const SideTaps<V> side = segmented ? SideTaps<V>(x0 + i, g.W, dil, rt.lpr, xs, V * rt.lpr)
+                                                       : SideTaps<V>(min(x0 + i, g.W - 1), g.W, dil, rt.lpr);
+                    float ra[NPQ][4];
 #pragma unroll
-                for (int co = 0; co < WOUT; co++)
+                    for (int pq = 0; pq < NPQ; pq++) {
+                        const float *srow = S + (size_t)(co * NPQ + pq) * rs;
+                        ra[pq][0] = srow[side.i0a];
+                        ra[pq][1] = srow[side.i0b];
+                        ra[pq][2] = srow[side.i2a];
+                        ra[pq][3] = srow[side.i2b];
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                     for (int pq = 0; pq < NPQ; pq++) {
                         const int r = co * NPQ + pq;   // staged row; its three taps are rows 3 r .. 3 r + 2 of tv
-                        tv[r * 3 + 0][i] = (side.m0a ? ra[r][0] : 0.f) + (side.m0b ? ra[r][1] : 0.f);
+                        tv[r * 3 + 0][i] = (side.m0a ? ra[pq][0] : 0.f) + (side.m0b ? ra[pq][1] : 0.f);
                         tv[r * 3 + 1][i] = own[co][pq][i];
-                        tv[r * 3 + 2][i] = (side.m2a ? ra[r][2] : 0.f) + (side.m2b ? ra[r][3] : 0.f);
+                        tv[r * 3 + 2][i] = (side.m2a ? ra[pq][2] : 0.f) + (side.m2b ? ra[pq][3] : 0.f);
                     }
-                __builtin_amdgcn_sched_barrier(0);
-            }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             __syncthreads();                      // the staged rows may be overwritten from here on
             // the wave's [row][voxel] tile; lanes past the image row hold finite values that meet zeros of x
 #pragma unroll
@@ -402,7 +405,7 @@ void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *_
         auto load_weights = [&](int ci, float (&w)[KR]) {
 #pragma unroll
             for (int co = 0; co < WOUT; co++) {
-                const float *kc = kw + (uint32_t)((co * g.C + ci) * K);
+                const float *kc = (co == 0 ? kw : kw1) + (uint32_t)(ci * K);
 #pragma unroll
                 for (int t = 0; t < K; t++) w[co * K + t] = kc[t];
             }
@@ -677,14 +680,22 @@ int choose_vec(const Geom &g, int vmax, const View<const float> &gy, const View<
     return 0;
 }
 
+// `pair`: the two output channels are two layers of a dense block (g.dil is then the larger of
+// their dilations, which is what the row segments' halo is sized for).
 template <int NDIM, int V, int NCB, int WOUT, bool LONG>
 hipError_t launch(const Geom &g, const View<const float> &gy, const View<const float> &x, const float *k,
                   const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws, hipStream_t s,
-                  ReduceJob *defer)
+                  ReduceJob *defer, const LayerPair *pair)
 {
     constexpr int K = Taps<NDIM>::K;
     Args a;
     a.g = g;
+    a.dil1 = 0;
+    if (pair) {
+        if (WOUT != 2) return hipErrorInvalidValue;
+        a.g.dil = pair->dil0;
+        a.dil1 = pair->dil1;
+    }
     a.sg = RowSegments{1, 0};
     make_row_teams(g, V, &a.rt, LONG ? &a.sg : nullptr);
     // a deferred reduction brings its own region for the partial sums (defer->part)
@@ -716,30 +727,36 @@ hipError_t launch(const Geom &g, const View<const float> &gy, const View<const f
     const int chunks = (g.C + NCB * kChanBlock - 1) / (NCB * kChanBlock);
     const size_t lds = lds_bytes<NDIM, V, NCB, WOUT>(a.rt, a.sg);
     if (lds > kMaxLdsBytes) return hipErrorInvalidConfiguration;   // excluded by fits()
+    // the weights of the second output channel follow those of the first, or are another layer's
+    const float *k1 = pair ? pair->k1 : k + (int64_t)g.C * K;
     hipLaunchKernelGGL((bwd_rows_fused<NDIM, V, NCB, WOUT, LONG>), dim3(rows, 1, chunks), dim3(a.rt.lpr * a.rt.rpw), lds, s, a,
-                       gy.p, x.p, gx.p, actp, k, part);
+                       gy.p, x.p, gx.p, actp, k, k1, part);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     const int64_t nk = (int64_t)WOUT * g.C * K;
     const int64_t ncols = nk + (a.want_bias ? WOUT : 0);
+    // columns [0, split) of the partial sums go to gk, [split, nk) to gk1
+    const int64_t split = pair ? (int64_t)g.C * K : nk;
+    float *gk1 = pair ? pair->gk1 : nullptr;
     if (defer) {
-        *defer = ReduceJob{part, gk, gb, nk, ncols, rows};
+        *defer = ReduceJob{part, gk, gb, nk, ncols, rows, gk1, split};
         return hipSuccess;
     }
-    hipLaunchKernelGGL(bwdk::reduce_columns, dim3((ncols + 3) / 4), dim3(256), 0, s, part, rows, nk, ncols, gk, gb);
+    hipLaunchKernelGGL(bwdk::reduce_columns, dim3((ncols + 3) / 4), dim3(256), 0, s, part, rows, nk, ncols, gk, gb, gk1,
+                       split);
     return hipGetLastError();
 }
 
 template <int NDIM, int V, int WOUT, bool LONG>
 hipError_t pick_ncb(const Geom &g, const View<const float> &gy, const View<const float> &x, const float *k,
                     const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws, hipStream_t s,
-                    ReduceJob *defer)
+                    ReduceJob *defer, const LayerPair *pair)
 {
     const int need = (g.C + kChanBlock - 1) / kChanBlock;
-    if (need <= 1) return launch<NDIM, V, 1, WOUT, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
-    if (need <= 2) return launch<NDIM, V, 2, WOUT, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
-    if (need <= 4) return launch<NDIM, V, 4, WOUT, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
-    return launch<NDIM, V, 8, WOUT, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
+    if (need <= 1) return launch<NDIM, V, 1, WOUT, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
+    if (need <= 2) return launch<NDIM, V, 2, WOUT, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
+    if (need <= 4) return launch<NDIM, V, 4, WOUT, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
+    return launch<NDIM, V, 8, WOUT, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
 }
 
 // Widest vector for two output channels (2D only): twice the gathered values per voxel must
@@ -777,7 +794,7 @@ Mode xkb_mode(const Geom &g, const View<const float> &gy, const View<const float
 template <int NDIM, bool LONG>
 hipError_t xkb_nd(const Geom &g, const View<const float> &gy, const View<const float> &x, const float *k,
                   const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws, hipStream_t s,
-                  ReduceJob *defer)
+                  ReduceJob *defer, const LayerPair *pair = nullptr)
 {
     // 3D: one voxel per lane keeps the 27 gathered values per voxel and the pipeline buffers in registers
     int vmax = knob(NDIM == 3 ? kKnobBwdkVec3d : kKnobBwdkVec2d, NDIM == 3 ? 1 : 4);
@@ -802,17 +819,17 @@ hipError_t xkb_nd(const Geom &g, const View<const float> &gy, const View<const f
         if (g.Wd == 2) {
             v = choose_vec<2>(g, std::min(vmax, kMaxVecTwoOutputs), gy, x, gx, LONG);
             if (v == 0) v = choose_vec<2>(g, kMaxVecTwoOutputs, gy, x, gx, LONG);
-            if (v == 2) return pick_ncb<2, 2, 2, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
-            if (v == 1) return pick_ncb<2, 1, 2, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
+            if (v == 2) return pick_ncb<2, 2, 2, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
+            if (v == 1) return pick_ncb<2, 1, 2, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
             return hipErrorInvalidConfiguration;
         }
-        if (v == 4) return pick_ncb<2, 4, 1, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
+        if (v == 4) return pick_ncb<2, 4, 1, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, nullptr);
     }
     if (g.Wd != 1) return hipErrorInvalidConfiguration;
     if constexpr (NDIM == 2) {
-        if (v == 2) return pick_ncb<2, 2, 1, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
+        if (v == 2) return pick_ncb<2, 2, 1, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, nullptr);
     }
-    if (v == 1) return pick_ncb<NDIM, 1, 1, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer);
+    if (v == 1) return pick_ncb<NDIM, 1, 1, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, nullptr);
     return hipErrorInvalidConfiguration;
 }
 

@@ -61,6 +61,7 @@ enum Knob {
     kKnobXcdRemap, kKnobBwdkVec2d, kKnobBwdkVec3d, kKnobBwdkBlocks,
     kKnobFwdVec2d, kKnobFwdVec3d, kKnobFwdSplit, kKnobFwdRows2d, kKnobBwdkRows, kKnobBlockFuse,
     kKnobBlockDefer, kKnobBwdkInterleave, kKnobBlockSnake, kKnobFwdClass3d, kKnobFwdLattice3d,
+    kKnobBlockPair,
     kKnobCount
 };
 int knob(Knob k, int dflt);
@@ -148,6 +149,17 @@ struct ReduceJob {
     float *gk, *gb;
     int64_t nk, ncols;
     int rows;
+    float *gk1;       // columns [split, nk) go here instead of to gk (a second layer's weight gradient)
+    int64_t split;    // nk where there is no second destination
+};
+// Two layers of a dense block as the two output channels of one fused backward pass over the
+// input channels they share: output channel 0 is the lower layer (dilation dil0, weights k,
+// weight gradient gk), output channel 1 the layer above it (dil1, k1, gk1; the first g.C of its
+// input channels).  The Geom's dilation is the larger of the two.
+struct LayerPair {
+    int dil0, dil1;
+    const float *k1;
+    float *gk1;
 };
 constexpr int kReduceBatch = 16;
 // One launch for up to kReduceBatch pending reductions; every column is added in the same
@@ -164,7 +176,7 @@ bool fast_backward_xkb_supported_3d(const Geom &g, const View<const float> &gy, 
                                     const View<float> &gx);
 hipError_t fast_backward_xkb_2d(const Geom &g, const View<const float> &gy, const View<const float> &x, const float *k,
                                 const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws,
-                                hipStream_t s, ReduceJob *defer);
+                                hipStream_t s, ReduceJob *defer, const LayerPair *pair = nullptr);
 hipError_t fast_backward_xkb_3d(const Geom &g, const View<const float> &gy, const View<const float> &x, const float *k,
                                 const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws,
                                 hipStream_t s, ReduceJob *defer);
@@ -172,7 +184,7 @@ hipError_t fast_backward_xkb_3d(const Geom &g, const View<const float> &gy, cons
 // not fit 32 bits; chosen by fast_backward_xkb_2d / _3d, not called directly
 hipError_t fast_backward_xkb_2d_long(const Geom &g, const View<const float> &gy, const View<const float> &x,
                                      const float *k, const View<float> &gx, const PostMask &pm, float *gk, float *gb,
-                                     float *ws, hipStream_t s, ReduceJob *defer);
+                                     float *ws, hipStream_t s, ReduceJob *defer, const LayerPair *pair = nullptr);
 hipError_t fast_backward_xkb_3d_long(const Geom &g, const View<const float> &gy, const View<const float> &x,
                                      const float *k, const View<float> &gx, const PostMask &pm, float *gk, float *gb,
                                      float *ws, hipStream_t s, ReduceJob *defer);

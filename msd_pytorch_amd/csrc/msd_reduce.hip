@@ -35,10 +35,14 @@ __global__ __launch_bounds__(256) void reduce_columns_batched(ReduceBatch b)
     for (int off = kWave / 2; off > 0; off >>= 1) s += __shfl_down(s, off, kWave);
     if (l == 0) {
         const int64_t nk = b.job[j].nk;
-        if (col < nk)
-            b.job[j].gk[col] += s;
-        else
+        if (col < nk) {
+            if (col < b.job[j].split)
+                b.job[j].gk[col] += s;
+            else
+                b.job[j].gk1[col - b.job[j].split] += s;
+        } else {
             b.job[j].gb[col - nk] += s;
+        }
     }
 }
 
@@ -58,7 +62,7 @@ hipError_t reduce_columns_batch(const ReduceJob *jobs, int n, hipStream_t s)
         b.first[i] = total;
         total += jobs[i].ncols;
     }
-    for (int i = n; i < kReduceBatch; i++) b.job[i] = ReduceJob{nullptr, nullptr, nullptr, 0, 0, 0};
+    for (int i = n; i < kReduceBatch; i++) b.job[i] = ReduceJob{nullptr, nullptr, nullptr, 0, 0, 0, nullptr, 0};
     for (int i = n; i <= kReduceBatch; i++) b.first[i] = total;
     b.n = n;
     if (total == 0) return hipSuccess;

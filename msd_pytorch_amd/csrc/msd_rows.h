@@ -163,20 +163,23 @@ inline size_t staged_floats(const RowTeams &rt, int wout)
 // the lane's own V values of every staged row in `own`.  Every lane of the
 // workgroup must call this; lanes outside the image (`act` false) stage zeros.
 // Ends with a workgroup barrier.
+// `dil1`: the dilation of the second output channel's taps where it has one of its own (two
+// layers of a dense block gathered in one pass); the layer's dilation otherwise.
 template <int NDIM, bool RELU, int WOUT, int V>
 __device__ __forceinline__ void stage_source_rows(const Geom &g, const RowTeams &rt, const View<const float> &out,
                                                   const View<const float> &gy, int b, int z, int y, int lane,
                                                   bool act, float *__restrict__ S,
-                                                  float (&own)[WOUT][RowTaps<NDIM>::NPQ][V])
+                                                  float (&own)[WOUT][RowTaps<NDIM>::NPQ][V], int dil1 = 0)
 {
     constexpr int NZ = Taps<NDIM>::NZ, NPQ = RowTaps<NDIM>::NPQ;
-    const AxisSources sz = NDIM == 3 ? adjoint_sources(z, g.D, g.dil) : single_source();
-    const AxisSources sy = adjoint_sources(y, g.H, g.dil);
     const int x0 = min(lane * V, g.W - V);   // lanes past the row read a valid address; their values are dropped
-    // rows whose taps fold: within dil of a y (or z) border
-    const bool folds = y < g.dil || y + g.dil >= g.H || (NDIM == 3 && (z < g.dil || z + g.dil >= g.D));
 #pragma unroll
     for (int co = 0; co < WOUT; co++) {
+        const int dil = (WOUT > 1 && co > 0 && dil1 > 0) ? dil1 : g.dil;
+        const AxisSources sz = NDIM == 3 ? adjoint_sources(z, g.D, dil) : single_source();
+        const AxisSources sy = adjoint_sources(y, g.H, dil);
+        // rows whose taps fold: within dil of a y (or z) border
+        const bool folds = y < dil || y + dil >= g.H || (NDIM == 3 && (z < dil || z + dil >= g.D));
         const float *gc = gy.p + (int64_t)b * gy.sb + (int64_t)co * gy.sc + x0;
         const float *oc = RELU ? out.p + (int64_t)b * out.sb + (int64_t)co * out.sc + x0 : nullptr;
         float s[NPQ][V];
@@ -235,21 +238,22 @@ template <int NDIM, int WOUT, int V>
 __device__ __forceinline__ void stage_source_segment(const Geom &g, const RowTeams &rt, const RowSegments &sg,
                                                      const View<const float> &gy, int b, int z, int y, int xs,
                                                      int lane, bool rowok, float *__restrict__ S,
-                                                     float (&own)[WOUT][RowTaps<NDIM>::NPQ][V])
+                                                     float (&own)[WOUT][RowTaps<NDIM>::NPQ][V], int dil1 = 0)
 {
     constexpr int NZ = Taps<NDIM>::NZ, NPQ = RowTaps<NDIM>::NPQ;
-    const AxisSources sz = NDIM == 3 ? adjoint_sources(z, g.D, g.dil) : single_source();
-    const AxisSources sy = adjoint_sources(y, g.H, g.dil);
-    const int rs = V * rt.lpr + sg.halo;         // floats per staged row
+    const int rs = V * rt.lpr + sg.halo;         // floats per staged row (the halo is sized for the larger dilation)
     const bool inrow = rowok && xs + lane * V < g.W;   // lanes past the row stage zeros ...
     const int x0 = min(xs + lane * V, g.W - V);        // ... read from a valid address
     const int h = lane;                          // halo element of this lane, if any
-    const int hx = h < g.dil ? xs - g.dil + h : xs + V * rt.lpr + (h - g.dil);
-    const bool hin = rowok && h < 2 * g.dil && hx >= 0 && hx < g.W;
-    const int hxc = min(max(hx, 0), g.W - 1);
-    const bool folds = y < g.dil || y + g.dil >= g.H || (NDIM == 3 && (z < g.dil || z + g.dil >= g.D));
 #pragma unroll
     for (int co = 0; co < WOUT; co++) {
+        const int dil = (WOUT > 1 && co > 0 && dil1 > 0) ? dil1 : g.dil;
+        const AxisSources sz = NDIM == 3 ? adjoint_sources(z, g.D, dil) : single_source();
+        const AxisSources sy = adjoint_sources(y, g.H, dil);
+        const int hx = h < dil ? xs - dil + h : xs + V * rt.lpr + (h - dil);
+        const bool hin = rowok && h < 2 * dil && hx >= 0 && hx < g.W;
+        const int hxc = min(max(hx, 0), g.W - 1);
+        const bool folds = y < dil || y + dil >= g.H || (NDIM == 3 && (z < dil || z + dil >= g.D));
         const float *gc = gy.p + (int64_t)b * gy.sb + (int64_t)co * gy.sc;
         float s[NPQ][V], sh[NPQ];
         auto add_row = [&](int pq, int cz, int cy, bool ok, bool first) {
@@ -288,7 +292,7 @@ __device__ __forceinline__ void stage_source_segment(const Geom &g, const RowTea
                 own[co][pq][i] = s[pq][i];
                 row[i * rt.lpr + lane] = s[pq][i];
             }
-            if (h < 2 * g.dil) row[V * rt.lpr + h] = sh[pq];
+            if (h < 2 * dil) row[V * rt.lpr + h] = sh[pq];
         }
     }
     __syncthreads();

@@ -140,7 +140,9 @@ def test_operators_under_a_forced_setting(cc, case):
 
 
 BLOCK_SETTINGS = [{"block.snake": 0}, {"block.snake": 1}, {"block.fuse": 0}, {"block.defer": 0},
-                  {"xcd_remap": 0}, {"bwdk.interleave": 0}, {"fwd.class3d": 0}, {"fwd.lattice3d": 44}]
+                  {"xcd_remap": 0}, {"bwdk.interleave": 0}, {"fwd.class3d": 0}, {"fwd.lattice3d": 44},
+                  {"block.pair": 0}, {"block.pair": 1}, {"block.pair": 1, "block.defer": 0},
+                  {"block.pair": 1, "block.snake": 0}]
 
 
 @pytest.mark.parametrize("settings", BLOCK_SETTINGS, ids=lambda s: ",".join("%s=%d" % kv for kv in s.items()))
@@ -148,3 +150,49 @@ BLOCK_SETTINGS = [{"block.snake": 0}, {"block.snake": 1}, {"block.fuse": 0}, {"b
 def test_block_under_a_forced_setting(ndim, size, settings):
     with tuning(settings):
         check_block(ndim, size, 2, 1, 19, 2)
+
+
+# The backward pass of a 2D block of one-channel layers takes the layers two at a time (the
+# pair's second launch gathers two output gradients with two dilations in one pass over the
+# channels both layers read).  Cases: equal and very different dilations in a pair, dilations
+# that fold on both sides of a small image, odd and even depths (a layer left over at the
+# bottom), more than one input channel, rows that one workgroup covers (256, 512 voxels), rows
+# cut into segments (1280, 2050: not a multiple of four) and short odd rows.
+PAIR_BLOCKS = [
+    # (size, c_in, depth, batch, dilations)
+    ((21, 256), 1, 6, 2, [1, 10, 2, 9, 3, 8]),
+    ((21, 256), 3, 7, 1, [5, 5, 5, 1, 1, 7, 2]),
+    ((12, 512), 2, 5, 1, [12, 1, 11, 2, 6]),
+    ((9, 1280), 1, 6, 1, [1, 4, 9, 2, 3, 7]),
+    ((7, 2050), 1, 4, 1, [3, 1, 6, 2]),
+    ((33, 70), 2, 9, 2, [1, 2, 3, 4, 5, 6, 7, 8, 9]),
+    ((40, 64), 1, 20, 1, None),
+]
+
+
+@pytest.mark.parametrize("pair", [1, 0], ids=["paired", "single"])
+@pytest.mark.parametrize("case", PAIR_BLOCKS, ids=lambda c: "x".join(map(str, c[0])) + "-d%d" % c[2])
+def test_block_backward_two_layers_at_a_time(case, pair):
+    size, c_in, depth, batch, dilations = case
+    with tuning({"block.pair": pair}):
+        check_block(2, size, c_in, 1, depth, batch, dilations=dilations, seed=11)
+
+
+def test_paired_and_single_backward_agree_when_the_input_needs_no_gradient():
+    # the model path: the block's input is data, so the lowest layer takes the weight-gradient
+    # kernel alone and the pairs start one layer higher
+    from msd_pytorch_amd.msd_block import msd_block
+    from parity import block_problem
+    from cases import rel_err
+    x, dil, bias, ws, g = block_problem(2, (19, 384), 1, 1, 8, 2, seed=5)
+    grads = {}
+    for pair in (0, 1):
+        with tuning({"block.pair": pair}):
+            bd = bias.cuda().requires_grad_(True)
+            wd = [w.cuda().requires_grad_(True) for w in ws]
+            out = msd_block(x.cuda(), dil, bd, *wd)
+            out.backward(g.cuda())
+            torch.cuda.synchronize()
+            grads[pair] = [bd.grad.clone()] + [w.grad.clone() for w in wd]
+    for a, b in zip(grads[0], grads[1]):
+        assert rel_err(a, b) <= 1e-5
