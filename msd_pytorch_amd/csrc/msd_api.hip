@@ -854,7 +854,9 @@ int block_pair_fused(const char *fn, const BlockArgs &a, int i, int64_t first, c
     gx1.p += c * gx.sc;
     gy1 = msd::View<const float>{gx.p + first * gx.sc, gx.sb, gx.sc, gx.sz, gx.sy, gx.sx};   // layer i's output gradient
     gy2 = msd::View<const float>{gx.p + c * gx.sc, gx.sb, gx.sc, gx.sz, gx.sy, gx.sx};       // layer i - 1's, then layer i's
-    if (!msd::fast_backward_xkb_supported(g1, gy1, x1, gx1) || !msd::fast_backward_xkb_supported(g2, gy2, x, gx))
+    const bool lean = msd::fast_backward_one_channel_supported_2d(g1, gy1, x1, gx1);
+    if ((!lean && !msd::fast_backward_xkb_supported(g1, gy1, x1, gx1)) ||
+        !msd::fast_backward_xkb_supported(g2, gy2, x, gx))
         return MSD_OK;
     MSD_TRY(check_workspace(fn, g1, sizeof(float), ws, ws_bytes));
     MSD_TRY(check_workspace(fn, g2, sizeof(float), ws, ws_bytes));
@@ -867,8 +869,11 @@ int block_pair_fused(const char *fn, const BlockArgs &a, int i, int64_t first, c
         msd::ReduceJob *job = nullptr;
         MSD_TRY(pending->next(fn, region, &job));
         ProfileScope scope(3, s);
-        const hipError_t e = msd::fast_backward_xkb(g1, gy1, x1, w_hi + c * K, gx1, pm, gk_hi + c * K, nullptr,
-                                                    (float *)ws, s, job);
+        const hipError_t e =
+            lean ? msd::fast_backward_one_channel_2d(g1, gy1, x1, w_hi + c * K, gx1, pm, gk_hi + c * K, (float *)ws, s,
+                                                     job)
+                 : msd::fast_backward_xkb(g1, gy1, x1, w_hi + c * K, gx1, pm, gk_hi + c * K, nullptr, (float *)ws, s,
+                                          job);
         if (e != hipSuccess) return hip_fail(fn, e);
         if (job) pending->taken(region);
     }

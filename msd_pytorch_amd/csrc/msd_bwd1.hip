@@ -1,0 +1,194 @@
+// Backward pass of one layer over ONE input channel, 2D, fp32: grad_input of that channel,
+// the nine weight gradients of that channel, and the channel's ReLU mask on the way out.
+//
+// The dense block's backward loop takes its layers two at a time (msd_api.hip): the upper
+// layer of a pair first has to finish the gradient of the channel the lower layer wrote, one
+// channel out of up to a hundred.  The fused kernel (msd_bwdxk_impl.h) does that too, but its
+// pipeline of 16-channel blocks on the matrix cores runs in full for the one channel (20 us at
+// 1024 x 1024); here the channel is four planes of memory traffic and 18 multiply-adds per
+// voxel on the vector pipe: the gather of msd_rows.h (the same one, so the same values), one
+// load of x and grad_input per lane, nine running sums per lane for the weight gradient,
+// reduced once per workgroup into a row of partial sums (fixed order; second pass as for the
+// other weight-gradient kernels).
+// Semantics: conv2d_backward_x.cu:109-208 and conv2d_backward_k.cu:61-112 of the reference,
+// restricted to one input channel.
+#include "msd_kernels.h"
+#include "msd_rows.h"
+
+namespace msd {
+namespace bwd1 {
+
+constexpr int kThreads = 256;
+constexpr int K = 9, NPQ = 3;
+
+struct Args {
+    Geom g;
+    RowTeams rt;
+    int ngroups, total_groups, tiles_per_wg;
+    int masked;
+    int gy_sb, gy_sy, x_sb, x_sy, gx_sb, gx_sy;
+};
+
+template <int V>
+__global__ __launch_bounds__(kThreads) void bwd_one_channel(const Args a, const float *__restrict__ gyp,
+                                                            const float *__restrict__ xp, float *__restrict__ gxp,
+                                                            const float *__restrict__ actp,
+                                                            const float *__restrict__ kw, float *__restrict__ part)
+{
+    extern __shared__ float lds[];
+    const Geom &g = a.g;
+    const RowTeams &rt = a.rt;
+    const int tid = threadIdx.x;
+    const int team = tid / rt.lpr, lane = tid % rt.lpr;
+    float *S = lds + (size_t)team * NPQ * V * rt.lpr;
+    float w[K];
+#pragma unroll
+    for (int t = 0; t < K; t++) w[t] = kw[t];     // uniform: scalar loads
+    float ksum[K];
+#pragma unroll
+    for (int t = 0; t < K; t++) ksum[t] = 0.f;
+    const int x0 = lane * V;
+    const int xc = min(x0, g.W - V);
+    const View<const float> none{nullptr, 0, 0, 0, 0, 0};
+    const View<const float> gyv{gyp, a.gy_sb, 0, 0, a.gy_sy, 1};
+
+    for (int ti = 0; ti < a.tiles_per_wg; ti++) {
+        const int grp = blockIdx.x + ti * gridDim.x;          // uniform
+        if (grp >= a.total_groups) break;
+        const int gi = grp % a.ngroups, b = grp / a.ngroups;
+        const int row = gi * rt.rpw + team;
+        const bool rowok = row < g.H;
+        const int y = rowok ? row : g.H - 1;
+        const bool act = rowok && x0 < g.W;
+        // the channel's own values are asked for first: their latency passes behind the gather
+        const int64_t xo = (int64_t)b * a.x_sb + (int64_t)y * a.x_sy + xc;
+        const int64_t go = (int64_t)b * a.gx_sb + (int64_t)y * a.gx_sy + xc;
+        float xv[V], gv[V], m[V];
+        load_vec<V>(xp + xo, xv);
+        load_vec<V>(gxp + go, gv);
+        if (a.masked) load_vec<V>(actp + go, m);   // uniform; the activations share grad_input's layout
+        float own[1][NPQ][V];
+        stage_source_rows<2, false, 1, V>(g, rt, none, gyv, b, 0, y, lane, act, S, own);
+        float tv[K][V];
+#pragma unroll
+        for (int i = 0; i < V; i++) {
+            const SideTaps<V> side(min(x0 + i, g.W - 1), g.W, g.dil, rt.lpr);
+#pragma unroll
+            for (int pq = 0; pq < NPQ; pq++) {
+                float t0, t2;
+                side.read(S + (size_t)pq * V * rt.lpr, t0, t2);
+                tv[pq * 3 + 0][i] = t0;
+                tv[pq * 3 + 1][i] = own[0][pq][i];
+                tv[pq * 3 + 2][i] = t2;
+            }
+        }
+        __syncthreads();                          // the staged rows may be overwritten from here on
+#pragma unroll
+        for (int i = 0; i < V; i++) {
+            float sum = w[0] * tv[0][i];
+#pragma unroll
+            for (int t = 1; t < K; t++) sum += w[t] * tv[t][i];
+            gv[i] += sum;
+            if (a.masked) gv[i] = 0.f < m[i] ? gv[i] : 0.f;
+        }
+        if (act) store_vec<V>(gxp + go, gv);
+        // lanes outside the image took their side taps from the last voxel's positions: their x counts as zero
+#pragma unroll
+        for (int i = 0; i < V; i++) xv[i] = act ? xv[i] : 0.f;
+#pragma unroll
+        for (int t = 0; t < K; t++)
+#pragma unroll
+            for (int i = 0; i < V; i++) ksum[t] += tv[t][i] * xv[i];
+    }
+
+    // the lanes of a wave by a fixed shuffle tree, then the waves in order
+    __syncthreads();
+    const int wave = tid / kWave, wl = tid % kWave, nwaves = blockDim.x / kWave;
+#pragma unroll
+    for (int t = 0; t < K; t++) {
+        float s = ksum[t];
+#pragma unroll
+        for (int off = kWave / 2; off > 0; off >>= 1) s += __shfl_down(s, off, kWave);
+        if (wl == 0) lds[wave * K + t] = s;
+    }
+    __syncthreads();
+    if (tid < K) {
+        float s = 0.f;
+        for (int v = 0; v < nwaves; v++) s += lds[v * K + tid];
+        part[(int64_t)tid * kMaxPartialRows + blockIdx.x] = s;
+    }
+}
+
+// Voxels per lane, or 0: rows of whole waves that one team of at most 256 lanes covers,
+// naturally aligned V-wide accesses in all three tensors.
+int choose_vec(const Geom &g, const View<const float> &gy, const View<const float> &x, const View<float> &gx,
+               RowTeams *rt)
+{
+    for (int v = 4; v >= 1; v /= 2) {
+        if (!rows_aligned(gy, g.W, v) || !rows_aligned(x, g.W, v) || !rows_aligned(gx, g.W, v)) continue;
+        if (!make_row_teams(g, v, rt)) continue;
+        if (rt->lpr % kWave != 0 || rt->lpr * rt->rpw > kThreads) continue;
+        return v;
+    }
+    return 0;
+}
+
+bool in_range(const Geom &g, const View<const float> &v)
+{
+    const int64_t lim = (int64_t)1 << 31;
+    return v.sx == 1 && v.sb < lim && v.sy < lim && (int64_t)(g.H - 1) * v.sy + g.W < lim;
+}
+
+}  // namespace bwd1
+
+bool fast_backward_one_channel_supported_2d(const Geom &g, const View<const float> &gy, const View<const float> &x,
+                                            const View<float> &gx)
+{
+    if (g.ndim != 2 || g.C != 1 || g.Wd != 1 || g.D != 1) return false;
+    const View<const float> gxc{gx.p, gx.sb, gx.sc, gx.sz, gx.sy, gx.sx};
+    if (!bwd1::in_range(g, gy) || !bwd1::in_range(g, x) || !bwd1::in_range(g, gxc)) return false;
+    RowTeams rt;
+    return bwd1::choose_vec(g, gy, x, gx, &rt) != 0;
+}
+
+hipError_t fast_backward_one_channel_2d(const Geom &g, const View<const float> &gy, const View<const float> &x,
+                                        const float *k, const View<float> &gx, const PostMask &pm, float *gk,
+                                        float *ws, hipStream_t s, ReduceJob *defer)
+{
+    bwd1::Args a;
+    a.g = g;
+    const int v = bwd1::choose_vec(g, gy, x, gx, &a.rt);
+    if (v == 0) return hipErrorInvalidConfiguration;
+    a.ngroups = (g.H + a.rt.rpw - 1) / a.rt.rpw;
+    const int64_t total = (int64_t)a.ngroups * g.B;
+    if (total > INT32_MAX) return hipErrorInvalidConfiguration;
+    a.total_groups = (int)total;
+    const int wgs = (int)std::min<int64_t>(total, kMaxPartialRows);
+    a.tiles_per_wg = (int)((total + wgs - 1) / wgs);
+    a.masked = pm.from < g.C;
+    a.gy_sb = (int)gy.sb; a.gy_sy = (int)gy.sy;
+    a.x_sb = (int)x.sb; a.x_sy = (int)x.sy;
+    a.gx_sb = (int)gx.sb; a.gx_sy = (int)gx.sy;
+    const float *actp = a.masked ? pm.act.p : x.p;
+    float *part = defer ? const_cast<float *>(defer->part) : ws + backward_k_mask_floats(g);
+    const size_t lds = std::max((size_t)a.rt.rpw * bwd1::NPQ * v * a.rt.lpr, (size_t)(bwd1::kThreads / kWave) * bwd1::K) *
+                       sizeof(float);
+    const dim3 grid(wgs), block(a.rt.lpr * a.rt.rpw);
+    if (v == 4)
+        hipLaunchKernelGGL(bwd1::bwd_one_channel<4>, grid, block, lds, s, a, gy.p, x.p, gx.p, actp, k, part);
+    else if (v == 2)
+        hipLaunchKernelGGL(bwd1::bwd_one_channel<2>, grid, block, lds, s, a, gy.p, x.p, gx.p, actp, k, part);
+    else
+        hipLaunchKernelGGL(bwd1::bwd_one_channel<1>, grid, block, lds, s, a, gy.p, x.p, gx.p, actp, k, part);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    const int64_t nk = bwd1::K;
+    if (defer) {
+        *defer = ReduceJob{part, gk, nullptr, nk, nk, wgs, nullptr, nk};
+        return hipSuccess;
+    }
+    const ReduceJob job{part, gk, nullptr, nk, nk, wgs, nullptr, nk};
+    return reduce_columns_batch(&job, 1, s);
+}
+
+}  // namespace msd

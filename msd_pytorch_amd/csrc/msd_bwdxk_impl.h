@@ -197,8 +197,9 @@ void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *_
     // channel loop, which has the scalar registers full of weights: kept, they are spilled to
     // lanes of a vector register, every use costs a vector instruction, and the register
     // allocation around them grows (3D, up to 32 channels per chunk: 142-150 -> 108-116 VGPRs,
-    // which is what lets a fourth workgroup share the CU).  2D is 2 % slower that way.
-    constexpr bool RELOAD = NDIM == 3;
+    // which is what lets a fourth workgroup share the CU).  The 2D instances with two output
+    // channels gain 1 % (245 -> 220 VGPRs at most); those with one are 2 % slower that way.
+    constexpr bool RELOAD = NDIM == 3 || WOUT == 2;
     typedef const __attribute__((address_space(4))) int *kernarg_words_t;
     kernarg_words_t kernarg = (kernarg_words_t)__builtin_amdgcn_kernarg_segment_ptr();
     for (int ti = 0; ti < a_.tiles_per_wg; ti++) {

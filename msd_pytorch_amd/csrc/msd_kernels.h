@@ -189,6 +189,14 @@ hipError_t fast_backward_xkb_3d_long(const Geom &g, const View<const float> &gy,
                                      const float *k, const View<float> &gx, const PostMask &pm, float *gk, float *gb,
                                      float *ws, hipStream_t s, ReduceJob *defer);
 
+// One layer over one input channel (2D): grad_input, the channel's nine weight gradients, its
+// ReLU mask (pm.from == 0) on the way out.  msd_bwd1.hip.
+bool fast_backward_one_channel_supported_2d(const Geom &g, const View<const float> &gy, const View<const float> &x,
+                                            const View<float> &gx);
+hipError_t fast_backward_one_channel_2d(const Geom &g, const View<const float> &gy, const View<const float> &x,
+                                        const float *k, const View<float> &gx, const PostMask &pm, float *gk,
+                                        float *ws, hipStream_t s, ReduceJob *defer);
+
 inline bool fast_backward_xkb_supported(const Geom &g, const View<const float> &gy, const View<const float> &x,
                                         const View<float> &gx)
 {
