@@ -99,6 +99,7 @@ INSTANCES = [
     ({"bwdk.rows": 0, "bwdk.vec3d": 4}, (1, 40, 1, (5, 6, 128), 2)),
     ({"bwdk.rows": 0, "bwdk.vec3d": 4}, (1, 70, 1, (5, 6, 128), 2)),
     ({"bwdk.vec2d": 1}, (1, 40, 1, (9, 128), 2)),
+    ({"bwdk.vec2d": 1}, (1, 70, 1, (9, 128), 2)),   # one voxel per lane, one output channel, > 64 channels
     ({"bwdk.vec2d": 2}, (1, 70, 1, (9, 128), 2)),
     ({"bwdk.vec2d": 4}, (1, 70, 1, (9, 256), 2)),
     ({"bwdk.vec3d": 1}, (1, 20, 1, (5, 6, 64), 2)),
@@ -166,6 +167,7 @@ PAIR_BLOCKS = [
     ((9, 1280), 1, 6, 1, [1, 4, 9, 2, 3, 7]),
     ((7, 2050), 1, 4, 1, [3, 1, 6, 2]),
     ((33, 70), 2, 9, 2, [1, 2, 3, 4, 5, 6, 7, 8, 9]),
+    ((20, 255), 1, 5, 1, [2, 7, 1, 4, 3]),          # odd rows: one voxel per lane in the one-channel step
     ((40, 64), 1, 20, 1, None),
 ]
 
