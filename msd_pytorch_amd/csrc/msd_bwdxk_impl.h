@@ -103,7 +103,10 @@ template <int NDIM, int V, int NCB, int WOUT, bool LONG> constexpr int pipeline_
 // voxels), and rows longer than a workgroup covers are cut into segments, staged with a halo of
 // `dil` values on either side.  It is a separate
 // instance because even its few extra scalar instructions per stage cost the plain one 1-4 %.
-template <int NDIM, int V, int NCB, int WOUT, bool LONG>
+// BIG (LONG instances only): the 64-bit channel bases and the loads from any address; without it
+// a LONG instance only cuts rows into segments and addresses like the plain one (whole groups of
+// four voxels, stacks below 2^30 values), which saves a fifth of a stage's instructions.
+template <int NDIM, int V, int NCB, int WOUT, bool LONG, bool BIG = LONG>
 __global__ __launch_bounds__(kThreads, (resident_per_cu<NDIM, V, NCB, WOUT, LONG>()))
 void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *__restrict__ xp,
                     float *__restrict__ gxp, const float *__restrict__ actp, const float *__restrict__ kw,
@@ -240,7 +243,7 @@ void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *_
         // channel's byte offset is a 32-bit product: three scalar instructions instead of seven)
         auto channel_base = [&](uint64_t base, int ci) {
             uint64_t p;
-            if constexpr (LONG)
+            if constexpr (BIG)
                 p = base + (uint64_t)((int64_t)ci * gsc * 4);
             else
                 p = base + (uint64_t)((uint32_t)ci * (uint32_t)gsc * 4u);
@@ -257,7 +260,7 @@ void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *_
             // (redefining the lane offset keeps its widening to 64 bits next to the loads, where
             // it is free; hoisted out of the loop it would make every address a vector addition)
             asm volatile("" : "+v"(goff));
-            if constexpr (LONG) {
+            if constexpr (BIG) {
                 const int cb0 = c0 + cb * kChanBlock;
                 const uint64_t xb = xbase + (uint64_t)(uint32_t)cb0 * (uint32_t)(4 * xsc);
                 const uint32_t xch = (uint32_t)min(mj, g.C - 1 - cb0) * (uint32_t)xsc + xrow;
@@ -375,7 +378,7 @@ void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *_
                 const int s = h * NSS + j;
                 const bool vok = rowok && kx + 16 * s < g.W;
                 const bool keep = vok && chok;
-                if constexpr (LONG) {
+                if constexpr (BIG) {
                     // rows need not be whole groups of four voxels here: the last group of a row
                     // was loaded from W - 4 (inside the row), `shift` voxels early; move its
                     // values down and fill with zeros
@@ -683,7 +686,7 @@ int choose_vec(const Geom &g, int vmax, const View<const float> &gy, const View<
 
 // `pair`: the two output channels are two layers of a dense block (g.dil is then the larger of
 // their dilations, which is what the row segments' halo is sized for).
-template <int NDIM, int V, int NCB, int WOUT, bool LONG>
+template <int NDIM, int V, int NCB, int WOUT, bool LONG, bool BIG = LONG>
 hipError_t launch(const Geom &g, const View<const float> &gy, const View<const float> &x, const float *k,
                   const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws, hipStream_t s,
                   ReduceJob *defer, const LayerPair *pair)
@@ -730,7 +733,7 @@ hipError_t launch(const Geom &g, const View<const float> &gy, const View<const f
     if (lds > kMaxLdsBytes) return hipErrorInvalidConfiguration;   // excluded by fits()
     // the weights of the second output channel follow those of the first, or are another layer's
     const float *k1 = pair ? pair->k1 : k + (int64_t)g.C * K;
-    hipLaunchKernelGGL((bwd_rows_fused<NDIM, V, NCB, WOUT, LONG>), dim3(rows, 1, chunks), dim3(a.rt.lpr * a.rt.rpw), lds, s, a,
+    hipLaunchKernelGGL((bwd_rows_fused<NDIM, V, NCB, WOUT, LONG, BIG>), dim3(rows, 1, chunks), dim3(a.rt.lpr * a.rt.rpw), lds, s, a,
                        gy.p, x.p, gx.p, actp, k, k1, part);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
@@ -748,16 +751,16 @@ hipError_t launch(const Geom &g, const View<const float> &gy, const View<const f
     return hipGetLastError();
 }
 
-template <int NDIM, int V, int WOUT, bool LONG>
+template <int NDIM, int V, int WOUT, bool LONG, bool BIG = LONG>
 hipError_t pick_ncb(const Geom &g, const View<const float> &gy, const View<const float> &x, const float *k,
                     const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws, hipStream_t s,
                     ReduceJob *defer, const LayerPair *pair)
 {
     const int need = (g.C + kChanBlock - 1) / kChanBlock;
-    if (need <= 1) return launch<NDIM, V, 1, WOUT, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
-    if (need <= 2) return launch<NDIM, V, 2, WOUT, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
-    if (need <= 4) return launch<NDIM, V, 4, WOUT, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
-    return launch<NDIM, V, 8, WOUT, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
+    if (need <= 1) return launch<NDIM, V, 1, WOUT, LONG, BIG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
+    if (need <= 2) return launch<NDIM, V, 2, WOUT, LONG, BIG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
+    if (need <= 4) return launch<NDIM, V, 4, WOUT, LONG, BIG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
+    return launch<NDIM, V, 8, WOUT, LONG, BIG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
 }
 
 // Widest vector for two output channels (2D only): twice the gathered values per voxel must
@@ -820,6 +823,17 @@ hipError_t xkb_nd(const Geom &g, const View<const float> &gy, const View<const f
         if (g.Wd == 2) {
             v = choose_vec<2>(g, std::min(vmax, kMaxVecTwoOutputs), gy, x, gx, LONG);
             if (v == 0) v = choose_vec<2>(g, kMaxVecTwoOutputs, gy, x, gx, LONG);
+            if constexpr (LONG) {
+                // rows that are only long (whole groups of four voxels, aligned, offsets within 32
+                // bits like the plain kernel asks): segments without the other LONG machinery
+                const View<const float> gxc{gx.p, gx.sb, gx.sc, gx.sz, gx.sy, gx.sx};
+                const bool segments_only = g.W % 4 == 0 && rows_aligned(x, g.W, 4) && x_offsets_fit(g, x, false) &&
+                                           x_offsets_fit(g, gxc, false);
+                if (segments_only && v == 2)
+                    return pick_ncb<2, 2, 2, true, false>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
+                if (segments_only && v == 1)
+                    return pick_ncb<2, 1, 2, true, false>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
+            }
             if (v == 2) return pick_ncb<2, 2, 2, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
             if (v == 1) return pick_ncb<2, 1, 2, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
             return hipErrorInvalidConfiguration;

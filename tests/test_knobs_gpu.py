@@ -123,6 +123,17 @@ INSTANCES = [
     ({"bwdx.vec3d": 4, "bwdx.unroll3d": 2}, (1, 5, 1, (3, 4, 1536), 3)),   # 3D rows of 384 lanes
     ({"bwdx.vec3d": 4, "bwdx.unroll3d": 4}, (1, 5, 1, (3, 4, 1536), 3)),
     ({"bwdx.vec3d": 4, "bwdx.unroll3d": 4}, (1, 5, 2, (3, 4, 768), 3)),
+    # two output channels, rows cut into segments but otherwise like the plain kernel's (whole
+    # groups of four voxels, aligned): the segment-only instances, by channel blocks and voxels per lane
+    ({}, (1, 9, 2, (5, 1280), 3)),
+    ({}, (1, 20, 2, (8, 1280), 7)),
+    ({}, (1, 40, 2, (4, 1280), 2)),
+    ({}, (1, 70, 2, (6, 1280), 5)),
+    ({"bwdk.vec2d": 1}, (1, 9, 2, (5, 1280), 3)),
+    ({"bwdk.vec2d": 1}, (1, 20, 2, (8, 1280), 7)),
+    ({"bwdk.vec2d": 1}, (1, 40, 2, (4, 1280), 2)),
+    ({"bwdk.vec2d": 1}, (1, 70, 2, (6, 1280), 5)),
+    ({}, (1, 20, 2, (5, 1026), 3)),                  # long rows of whole pairs only: the full LONG instance, two blocks
 ]
 
 
