@@ -76,6 +76,11 @@ struct Args {
     int dil1;            // two output channels: the dilation of the second one's taps (two layers in one pass)
 };
 
+// The waves' tiles share the LDS of the staged rows (two outputs at four voxels per lane: the
+// tiles alone are 79 KB).
+template <int NDIM, int V, int WOUT>
+constexpr bool tiles_over_staging() { return NDIM == 2 && V == 4 && WOUT == 2; }
+
 // Workgroups (of four waves) that are resident per CU.  The 3D kernel with one voxel per lane
 // (pipeline stages of 16 voxels, arguments read again per tile, row arithmetic on the scalar
 // pipe, see the tile loop) needs 94 to 118 registers with up to 64 channels per chunk: four
@@ -153,8 +158,13 @@ void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *_
     const bool segmented = SEG && a.sg.segs > 1;  // uniform
     const int rs = V * rt.lpr + (SEG ? a.sg.halo : 0);   // floats per staged row
     float *S = lds + (size_t)team * WOUT * NPQ * rs;
-    float *AT = lds + (size_t)rt.rpw * WOUT * NPQ * rs + (size_t)wave * ATile<NDIM, V, WOUT>::kFloats;
-    for (int i = wl; i < ASTRIDE; i += kWave) AT[KR * ASTRIDE + i] = 0.f;
+    // ALIAS: the waves' tiles lie over the staged rows (the rows are dead once gathered), which
+    // takes a workgroup-wide barrier more per tile and brings the instance within the LDS of
+    // two workgroups per CU
+    constexpr bool ALIAS = tiles_over_staging<NDIM, V, WOUT>();
+    float *AT = lds + (ALIAS ? 0 : (size_t)rt.rpw * WOUT * NPQ * rs) + (size_t)wave * ATile<NDIM, V, WOUT>::kFloats;
+    if constexpr (!ALIAS)
+        for (int i = wl; i < ASTRIDE; i += kWave) AT[KR * ASTRIDE + i] = 0.f;
 
     const int c0 = blockIdx.z * NCB * kChanBlock;
     const int c_end = min(g.C, c0 + NCB * kChanBlock);   // channels of this chunk end here
@@ -349,6 +359,8 @@ void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *_
                     __builtin_amdgcn_sched_barrier(0);
                 }
             __syncthreads();                      // the staged rows may be overwritten from here on
+            if constexpr (ALIAS)
+                for (int i = wl; i < ASTRIDE; i += kWave) AT[KR * ASTRIDE + i] = 0.f;
             // the wave's [row][voxel] tile; lanes past the image row hold finite values that meet zeros of x
 #pragma unroll
             for (int t = 0; t < KR; t++) store_vec<V>(AT + t * ASTRIDE + wl * V, tv[t]);
@@ -552,6 +564,7 @@ void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *_
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        if constexpr (ALIAS) __syncthreads();     // the next tile's staged rows overwrite every wave's tile
         // next row group
         if (a.group_step != 1 || SEG) {           // uniform
             grp += a.group_step;
@@ -631,13 +644,17 @@ template <int NDIM, int V, int NCB, int WOUT>
 size_t lds_bytes(const RowTeams &rt, const RowSegments &sg)
 {
     constexpr int TG = (WOUT * Taps<NDIM>::K + 15) / 16;
-    const size_t main_loop = ((size_t)rt.rpw * WOUT * RowTaps<NDIM>::NPQ * (V * rt.lpr + sg.halo) +
-                              (size_t)kWaves * ATile<NDIM, V, WOUT>::kFloats) * 4;
+    const size_t staged = (size_t)rt.rpw * WOUT * RowTaps<NDIM>::NPQ * (V * rt.lpr + sg.halo) * 4;
+    const size_t tiles = (size_t)kWaves * ATile<NDIM, V, WOUT>::kFloats * 4;
+    const size_t main_loop = tiles_over_staging<NDIM, V, WOUT>() ? std::max(staged, tiles) : staged + tiles;
     const size_t epilogue = (size_t)kWaves * NCB * TG * 4 * kWave * 4;
     return std::max(main_loop, epilogue);
 }
 
 constexpr size_t kMaxLdsBytes = 64 * 1024;
+// what the instances with tiles over the staged rows ask for (an opt-in per kernel): two such
+// workgroups fill the 160 KB of a CU
+constexpr size_t kMaxLdsBytesAsked = 80 * 1024;
 
 // Strides and in-plane offsets fit the kernel's 32-bit arithmetic.
 template <typename T>
@@ -665,9 +682,10 @@ bool fits(const Geom &g, int V, const View<const float> &gy, const View<const fl
     // opting in to more (3D rows of 512 voxels at two voxels per lane would take 77 KB: such
     // rows are cut into segments by the LONG instances instead)
     const size_t kr = (size_t)g.Wd * Taps<NDIM>::K + 1;
-    const size_t main_loop = ((size_t)rt.rpw * g.Wd * RowTaps<NDIM>::NPQ * (V * rt.lpr + sg.halo) +
-                              (size_t)kWaves * kr * (kWave * V + 4)) * 4;
-    if (main_loop > kMaxLdsBytes) return false;
+    const size_t staged = (size_t)rt.rpw * g.Wd * RowTaps<NDIM>::NPQ * (V * rt.lpr + sg.halo) * 4;
+    const size_t tiles = (size_t)kWaves * kr * (kWave * V + 4) * 4;
+    const bool over = NDIM == 2 && V == 4 && g.Wd == 2;   // tiles_over_staging()
+    if ((over ? std::max(staged, tiles) : staged + tiles) > (over ? kMaxLdsBytesAsked : kMaxLdsBytes)) return false;
     return rows_aligned(gy, g.W, V) && rows_aligned(gx, g.W, V);
 }
 
@@ -730,7 +748,13 @@ hipError_t launch(const Geom &g, const View<const float> &gy, const View<const f
     a.want_bias = gb != nullptr;
     const int chunks = (g.C + NCB * kChanBlock - 1) / (NCB * kChanBlock);
     const size_t lds = lds_bytes<NDIM, V, NCB, WOUT>(a.rt, a.sg);
-    if (lds > kMaxLdsBytes) return hipErrorInvalidConfiguration;   // excluded by fits()
+    constexpr bool kAsks = tiles_over_staging<NDIM, V, WOUT>();
+    if (lds > (kAsks ? kMaxLdsBytesAsked : kMaxLdsBytes)) return hipErrorInvalidConfiguration;   // excluded by fits()
+    if (kAsks && lds > kMaxLdsBytes) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&bwd_rows_fused<NDIM, V, NCB, WOUT, LONG, BIG>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLdsBytesAsked);
+        if (e != hipSuccess) return e;
+    }
     // the weights of the second output channel follow those of the first, or are another layer's
     const float *k1 = pair ? pair->k1 : k + (int64_t)g.C * K;
     hipLaunchKernelGGL((bwd_rows_fused<NDIM, V, NCB, WOUT, LONG, BIG>), dim3(rows, 1, chunks), dim3(a.rt.lpr * a.rt.rpw), lds, s, a,
@@ -766,6 +790,8 @@ hipError_t pick_ncb(const Geom &g, const View<const float> &gy, const View<const
 // Widest vector for two output channels (2D only): twice the gathered values per voxel must
 // still fit the registers beside the pipeline buffers.
 constexpr int kMaxVecTwoOutputs = 2;
+// ... four in the plain kernel, whose tiles lie over the staged rows
+constexpr int kMaxVecTwoOutputsPlain = 4;
 
 // Lane offsets into x fit 32 bits: they span the whole stack in the plain kernel, one block
 // of 16 channels in the LONG one.  The plain kernel asks the same of grad_input (its channel
@@ -788,7 +814,9 @@ Mode xkb_mode(const Geom &g, const View<const float> &gy, const View<const float
     if (!small_strides(g, gy) || !small_strides(g, x) || !small_strides(g, gx)) return kUnsupported;
     const int vmax = g.Wd == 2 ? kMaxVecTwoOutputs : 4;
     const View<const float> gxc{gx.p, gx.sb, gx.sc, gx.sz, gx.sy, gx.sx};
-    if (x_offsets_fit(g, x, false) && x_offsets_fit(g, gxc, false) && choose_vec<NDIM>(g, vmax, gy, x, gx, false) != 0)
+    const int vmax_plain = g.Wd == 2 ? kMaxVecTwoOutputsPlain : 4;
+    if (x_offsets_fit(g, x, false) && x_offsets_fit(g, gxc, false) &&
+        choose_vec<NDIM>(g, vmax_plain, gy, x, gx, false) != 0)
         return kPlain;
     if (x_offsets_fit(g, x, true) && choose_vec<NDIM>(g, vmax, gy, x, gx, true) != 0) return kLong;
     return kUnsupported;
@@ -808,7 +836,7 @@ hipError_t xkb_nd(const Geom &g, const View<const float> &gy, const View<const f
         // wins, else the one with the most tiles (256 x 256, 100 channels: 58 -> 39 us).
         int best = 0;
         int64_t best_tiles = 0;
-        for (int v = g.Wd == 2 ? kMaxVecTwoOutputs : 4; v >= 1; v /= 2) {
+        for (int v = g.Wd == 2 ? kMaxVecTwoOutputsPlain : 4; v >= 1; v /= 2) {
             RowTeams rt;
             if (!fits<NDIM>(g, v, gy, x, gx, LONG) || !make_row_teams(g, v, &rt)) continue;
             const int64_t tiles = (int64_t)g.B * ((rt.nrows + rt.rpw - 1) / rt.rpw);
@@ -821,19 +849,24 @@ hipError_t xkb_nd(const Geom &g, const View<const float> &gy, const View<const f
     if (v == 0) v = choose_vec<NDIM>(g, 4, gy, x, gx, LONG);
     if constexpr (NDIM == 2) {
         if (g.Wd == 2) {
-            v = choose_vec<2>(g, std::min(vmax, kMaxVecTwoOutputs), gy, x, gx, LONG);
-            if (v == 0) v = choose_vec<2>(g, kMaxVecTwoOutputs, gy, x, gx, LONG);
+            constexpr int vmax2 = LONG ? kMaxVecTwoOutputs : kMaxVecTwoOutputsPlain;
+            v = choose_vec<2>(g, std::min(vmax, vmax2), gy, x, gx, LONG);
+            if (v == 0) v = choose_vec<2>(g, vmax2, gy, x, gx, LONG);
             if constexpr (LONG) {
                 // rows that are only long (whole groups of four voxels, aligned, offsets within 32
                 // bits like the plain kernel asks): segments without the other LONG machinery
                 const View<const float> gxc{gx.p, gx.sb, gx.sc, gx.sz, gx.sy, gx.sx};
                 const bool segments_only = g.W % 4 == 0 && rows_aligned(x, g.W, 4) && x_offsets_fit(g, x, false) &&
                                            x_offsets_fit(g, gxc, false);
+                if (segments_only && vmax >= 4 && choose_vec<2>(g, 4, gy, x, gx, true) == 4)
+                    return pick_ncb<2, 4, 2, true, false>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
                 if (segments_only && v == 2)
                     return pick_ncb<2, 2, 2, true, false>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
                 if (segments_only && v == 1)
                     return pick_ncb<2, 1, 2, true, false>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
             }
+            if constexpr (!LONG)
+                if (v == 4) return pick_ncb<2, 4, 2, false>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
             if (v == 2) return pick_ncb<2, 2, 2, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
             if (v == 1) return pick_ncb<2, 1, 2, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
             return hipErrorInvalidConfiguration;

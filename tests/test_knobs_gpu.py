@@ -118,6 +118,7 @@ INSTANCES = [
     ({"fwd.vec2d": 1}, (1, 6, 2, (9, 128), 2)),
     ({"bwdk.vec2d": 2}, (1, 9, 2, (9, 256), 2)),
     ({"bwdk.vec2d": 2}, (1, 70, 2, (9, 256), 3)),
+    ({"bwdk.vec2d": 2}, (1, 20, 2, (9, 256), 3)),
     ({"bwdk.vec2d": 1}, (1, 20, 1, (9, 128), 2)),
     ({"bwdx.vec2d": 1, "bwdx.unroll2d": 4}, (1, 6, 2, (9, 128), 2)),
     ({"bwdx.vec3d": 4, "bwdx.unroll3d": 2}, (1, 5, 1, (3, 4, 1536), 3)),   # 3D rows of 384 lanes
@@ -129,11 +130,25 @@ INSTANCES = [
     ({}, (1, 20, 2, (8, 1280), 7)),
     ({}, (1, 40, 2, (4, 1280), 2)),
     ({}, (1, 70, 2, (6, 1280), 5)),
+    ({}, (2, 20, 2, (10, 4096), 9)),
+    ({"bwdk.vec2d": 2}, (1, 9, 2, (5, 1280), 3)),
+    ({"bwdk.vec2d": 2}, (1, 20, 2, (8, 1280), 7)),
+    ({"bwdk.vec2d": 2}, (1, 40, 2, (4, 1280), 2)),
+    ({"bwdk.vec2d": 2}, (1, 70, 2, (6, 1280), 5)),
     ({"bwdk.vec2d": 1}, (1, 9, 2, (5, 1280), 3)),
     ({"bwdk.vec2d": 1}, (1, 20, 2, (8, 1280), 7)),
     ({"bwdk.vec2d": 1}, (1, 40, 2, (4, 1280), 2)),
     ({"bwdk.vec2d": 1}, (1, 70, 2, (6, 1280), 5)),
     ({}, (1, 20, 2, (5, 1026), 3)),                  # long rows of whole pairs only: the full LONG instance, two blocks
+    # two output channels at four voxels per lane (the waves' tiles lie over the staged rows in
+    # LDS): rows of one to four waves, one to four rows per workgroup, by channel blocks
+    ({}, (1, 9, 2, (5, 1024), 3)),
+    ({}, (2, 20, 2, (7, 1024), 6)),
+    ({}, (1, 40, 2, (4, 768), 2)),
+    ({}, (1, 70, 2, (6, 1024), 5)),
+    ({"bwdk.vec2d": 4}, (1, 20, 2, (9, 512), 8)),
+    ({"bwdk.vec2d": 4}, (2, 40, 2, (10, 256), 1)),
+    ({"bwdk.vec2d": 4}, (1, 100, 2, (13, 256), 12)),
 ]
 
 
@@ -169,7 +184,8 @@ def test_block_under_a_forced_setting(ndim, size, settings):
 # channels both layers read).  Cases: equal and very different dilations in a pair, dilations
 # that fold on both sides of a small image, odd and even depths (a layer left over at the
 # bottom), more than one input channel, rows that one workgroup covers (256, 512 voxels), rows
-# cut into segments (1280, 2050: not a multiple of four) and short odd rows.
+# cut into segments (1280, 2050: not a multiple of four), rows of 768 and 1024 voxels (four per
+# lane) and short odd rows.
 PAIR_BLOCKS = [
     # (size, c_in, depth, batch, dilations)
     ((21, 256), 1, 6, 2, [1, 10, 2, 9, 3, 8]),
@@ -177,6 +193,8 @@ PAIR_BLOCKS = [
     ((12, 512), 2, 5, 1, [12, 1, 11, 2, 6]),
     ((9, 1280), 1, 6, 1, [1, 4, 9, 2, 3, 7]),
     ((7, 2050), 1, 4, 1, [3, 1, 6, 2]),
+    ((11, 1024), 1, 7, 1, [1, 10, 2, 9, 3, 8, 4]),  # four voxels per lane in the pair's pass
+    ((6, 768), 2, 4, 2, [5, 1, 2, 5]),
     ((33, 70), 2, 9, 2, [1, 2, 3, 4, 5, 6, 7, 8, 9]),
     ((20, 255), 1, 5, 1, [2, 7, 1, 4, 3]),          # odd rows: one voxel per lane in the one-channel step
     ((40, 64), 1, 20, 1, None),
