@@ -17,9 +17,9 @@ const char *const kKnobNames[kKnobCount] = {
     "xcd_remap", "bwdk.vec2d", "bwdk.vec3d", "bwdk.blocks",
     "fwd.vec2d", "fwd.vec3d", "fwd.split", "fwd.rows2d", "bwdk.rows", "block.fuse",
     "block.defer", "bwdk.interleave", "block.snake", "fwd.class3d", "fwd.lattice3d",
-    "block.pair",
+    "block.pair", "block.triple",
 };
-static_assert(kKnobBlockPair + 1 == kKnobCount, "one name per knob, in the order of the enum");
+static_assert(kKnobBlockTriple + 1 == kKnobCount, "one name per knob, in the order of the enum");
 int g_knobs[kKnobCount];
 // every knob starts at "library default"
 const bool g_knobs_ready = [] {
@@ -721,10 +721,11 @@ int64_t block_layer_workspace(int dtype, int ndim, int64_t batch, int64_t c_in, 
         if (widths[i] <= 0) return -1;
         int64_t n = msd_workspace_bytes(dtype, ndim, batch, total, widths[i], spatial);
         if (n < 0) return -1;
-        if (i + 1 < depth && ndim == 2 && widths[i] == 1 && widths[i + 1] == 1) {
-            // this layer and the one above it may run as the two output channels of one pass
-            const int64_t n2 = msd_workspace_bytes(dtype, ndim, batch, total, 2, spatial);
-            n = n2 > n ? n2 : n;
+        for (int up = 1; up < msd::kMaxLayerGroup; up++) {
+            // this layer and the one or two above it may run as the output channels of one pass
+            if (ndim != 2 || i + up >= depth || widths[i + up] != 1 || widths[i] != 1) break;
+            const int64_t nup = msd_workspace_bytes(dtype, ndim, batch, total, up + 1, spatial);
+            n = nup > n ? nup : n;
         }
         need = n > need ? n : need;
         total += widths[i];
@@ -810,89 +811,126 @@ int block_layer_fused(const char *fn, const BlockArgs &a, int i, int64_t first, 
     return MSD_OK;
 }
 
-// Two layers of the block backward pass, i and i - 1 (2D, one output channel each), in two
-// launches instead of two full passes.  Layer i's inputs are the channels [0, first), layer
-// i - 1's the channels [0, first - 1); channel c = first - 1 is layer i - 1's output.
-//   1. layer i alone on channel c: its grad_input contribution completes that channel's
-//      gradient (masked with the channel's activation on the way out: it is layer i - 1's
-//      output gradient from here on), plus the nine weight gradients of that channel;
-//   2. both layers on the channels [0, c) as the two output channels of ONE pass of the fused
+// A group of n = 2 or 3 layers of the block backward pass, i down to i - n + 1 (2D, one output
+// channel each), in n launches instead of n full passes.  Layer i's inputs are the channels
+// [0, first), those of the lowest layer of the group the channels [0, c), c = first - (n - 1);
+// channel first - j is layer i - j's output.
+//   1. the top j layers of the group on channel first - j alone, for j = 1 .. n - 1: their
+//      grad_input contributions complete that channel's gradient (masked with the channel's
+//      activation on the way out: it is layer i - j's output gradient from here on), plus the
+//      nine weight gradients of that channel per layer;
+//   2. all n layers on the channels [0, c) as the output channels of ONE pass of the fused
 //      kernel (each with its own dilation and weights): every channel of the input and of
-//      grad_input is moved once for the two layers, and both bias gradients are formed there.
+//      grad_input is moved once for the n layers, and their bias gradients are formed there.
 // *done is false (and nothing was launched) when the case is not covered.
-bool pair_candidate(const BlockArgs &a, int i, bool need_input_grad)
+bool group_candidate(const BlockArgs &a, int i, int n, bool need_input_grad)
 {
-    return a.dtype == MSD_F32 && a.ndim == 2 && g_kernel_path == 0 && i >= 1 && a.widths[i] == 1 &&
-           a.widths[i - 1] == 1 && (i - 1 > 0 || need_input_grad) && msd::knob(msd::kKnobBlockFuse, 1) &&
+    if (a.dtype != MSD_F32 || a.ndim != 2 || g_kernel_path != 0 || i - (n - 1) < 0) return false;
+    for (int j = 0; j < n; j++)
+        if (a.widths[i - j] != 1) return false;
+    return (i - (n - 1) > 0 || need_input_grad) && msd::knob(msd::kKnobBlockFuse, 1) &&
            msd::knob(msd::kKnobBlockPair, 1);
 }
 
-int block_pair_fused(const char *fn, const BlockArgs &a, int i, int64_t first, const void *stack,
-                     const int64_t *stack_strides, void *grads, const int64_t *grads_strides,
-                     const void *const *weights, void *const *grad_weights, void *gb_lower, void *ws, int64_t ws_bytes,
-                     hipStream_t s, DeferredReductions *pending, bool *masked, bool *done)
+// Layers to take together from layer i down, most first.  Three where the shared pass is over
+// enough channels to gain from it (its tiles cost more to set up than a pair's), or wherever
+// possible when asked for ("block.triple" 1; 0: never).
+int group_sizes(const BlockArgs &a, int i, int64_t first, bool need_input_grad, int (&sizes)[2])
+{
+    int m = 0;
+    const int triple = msd::knob(msd::kKnobBlockTriple, -1);
+    constexpr int64_t kTripleFromChannels = 32;
+    if (triple != 0 && group_candidate(a, i, 3, need_input_grad) && (triple > 0 || first - 2 >= kTripleFromChannels))
+        sizes[m++] = 3;
+    if (group_candidate(a, i, 2, need_input_grad)) sizes[m++] = 2;
+    return m;
+}
+
+int block_group_fused(const char *fn, const BlockArgs &a, int i, int n, int64_t first, const void *stack,
+                      const int64_t *stack_strides, void *grads, const int64_t *grads_strides,
+                      const void *const *weights, void *const *grad_weights, void *gb_lowest, void *ws,
+                      int64_t ws_bytes, hipStream_t s, DeferredReductions *pending, int pass_no, bool *masked,
+                      bool *done)
 {
     *done = false;
-    if (!grad_weights[i] || !grad_weights[i - 1] || !gb_lower) return MSD_OK;
-    const int64_t c = first - 1;                  // channels below both layers; index of layer i - 1's output
-    const int d_hi = (int)a.dilations[i], d_lo = (int)a.dilations[i - 1];
+    if (n < 2 || n > msd::kMaxLayerGroup || !gb_lowest) return MSD_OK;
+    for (int j = 0; j < n; j++)
+        if (!grad_weights[i - j]) return MSD_OK;
+    const int lo = i - (n - 1);                   // lowest layer of the group
+    const int64_t c = first - (n - 1);            // channels below all layers of the group
     constexpr int K = 9;
-    msd::Geom g1, g2;
-    MSD_TRY(make_geom(fn, a.dtype, a.ndim, a.batch, 1, 1, a.spatial, d_hi, true, &g1));
-    MSD_TRY(make_geom(fn, a.dtype, a.ndim, a.batch, c, 2, a.spatial, d_hi > d_lo ? d_hi : d_lo, true, &g2));
-    msd::View<const float> x, x1, gy1, gy2;
-    msd::View<float> gx, gx1;
+    msd::View<const float> x;
+    msd::View<float> gx;
     MSD_TRY(make_view(fn, "input", a.ndim, stack, stack_strides, &x));
     MSD_TRY(make_view(fn, "grad_input", a.ndim, grads, grads_strides, &gx));
     // the activations are read through grad_input's addressing: same strides and alignment
     const bool same_layout = x.sb == gx.sb && x.sc == gx.sc && x.sz == gx.sz && x.sy == gx.sy &&
                              reinterpret_cast<uintptr_t>(x.p) % 16 == reinterpret_cast<uintptr_t>(gx.p) % 16;
     if (!same_layout) return MSD_OK;
-    x1 = x;
-    x1.p += c * x.sc;
-    gx1 = gx;
-    gx1.p += c * gx.sc;
-    gy1 = msd::View<const float>{gx.p + first * gx.sc, gx.sb, gx.sc, gx.sz, gx.sy, gx.sx};   // layer i's output gradient
-    gy2 = msd::View<const float>{gx.p + c * gx.sc, gx.sb, gx.sc, gx.sz, gx.sy, gx.sx};       // layer i - 1's, then layer i's
-    const bool lean = msd::fast_backward_one_channel_supported_2d(g1, gy1, x1, gx1);
-    if ((!lean && !msd::fast_backward_xkb_supported(g1, gy1, x1, gx1)) ||
-        !msd::fast_backward_xkb_supported(g2, gy2, x, gx))
-        return MSD_OK;
-    MSD_TRY(check_workspace(fn, g1, sizeof(float), ws, ws_bytes));
-    MSD_TRY(check_workspace(fn, g2, sizeof(float), ws, ws_bytes));
-    const float *w_hi = (const float *)weights[i], *w_lo = (const float *)weights[i - 1];
-    float *gk_hi = (float *)grad_weights[i], *gk_lo = (float *)grad_weights[i - 1];
-    {
-        // 1. channel c, layer i; the channel is an output of the layer below: masked on the way out
-        const msd::PostMask pm{0, x1};
-        const int64_t region = partial_region_floats(a.ndim, 1, 1);
-        msd::ReduceJob *job = nullptr;
-        MSD_TRY(pending->next(fn, region, &job));
-        ProfileScope scope(3, s);
-        const hipError_t e =
-            lean ? msd::fast_backward_one_channel_2d(g1, gy1, x1, w_hi + c * K, gx1, pm, gk_hi + c * K, (float *)ws, s,
-                                                     job)
-                 : msd::fast_backward_xkb(g1, gy1, x1, w_hi + c * K, gx1, pm, gk_hi + c * K, nullptr, (float *)ws, s,
-                                          job);
-        if (e != hipSuccess) return hip_fail(fn, e);
-        if (job) pending->taken(region);
-    }
-    {
-        // 2. channels [0, c), both layers; the outputs of layer i - 2 are complete with this update
-        msd::PostMask pm{g2.C, {nullptr, 0, 0, 0, 0, 0}};
-        *masked = false;
-        if (i - 2 >= 0) {
-            pm = msd::PostMask{(int)(c - a.widths[i - 2]), x};
-            *masked = true;
+    // launch j = 1 .. n - 1: the top j layers on channel first - j; launch n: all on [0, c)
+    struct Step {
+        msd::Geom g;
+        msd::View<const float> gy, x;
+        msd::View<float> gx;
+        msd::LayerGroup group;
+        const float *k;
+        float *gk;
+        bool lean;
+    } steps[msd::kMaxLayerGroup];
+    for (int j = 1; j <= n; j++) {
+        Step &st = steps[j - 1];
+        const bool shared = j == n;               // the pass over the channels all layers read
+        const int64_t ch = shared ? 0 : first - j, chans = shared ? c : 1;
+        const int bottom = i - j + 1;             // output channel 0 of this launch
+        int dmax = 0;
+        st.group.n = j;
+        for (int q = 0; q < j; q++) {
+            st.group.dil[q] = (int)a.dilations[bottom + q];
+            dmax = st.group.dil[q] > dmax ? st.group.dil[q] : dmax;
+            if (q > 0) {
+                st.group.k_up[q - 1] = (const float *)weights[bottom + q] + ch * K;
+                st.group.gk_up[q - 1] = (float *)grad_weights[bottom + q] + ch * K;
+            }
         }
-        const int64_t region = partial_region_floats(a.ndim, c, 2);
+        st.k = (const float *)weights[bottom] + ch * K;
+        st.gk = (float *)grad_weights[bottom] + ch * K;
+        MSD_TRY(make_geom(fn, a.dtype, a.ndim, a.batch, chans, j, a.spatial, dmax, true, &st.g));
+        st.x = x;
+        st.x.p += ch * x.sc;
+        st.gx = gx;
+        st.gx.p += ch * gx.sc;
+        // the output gradients of the launch's layers: the channels above the highest one it updates
+        const int64_t gy_ch = shared ? c : ch + 1;
+        st.gy = msd::View<const float>{gx.p + gy_ch * gx.sc, gx.sb, gx.sc, gx.sz, gx.sy, gx.sx};
+        st.lean = !shared && msd::fast_backward_one_channel_supported_2d(st.g, st.gy, st.x, st.gx);
+        if (!st.lean && !msd::fast_backward_xkb_supported(st.g, st.gy, st.x, st.gx)) return MSD_OK;
+        MSD_TRY(check_workspace(fn, st.g, sizeof(float), ws, ws_bytes));
+    }
+    for (int j = 1; j <= n; j++) {
+        Step &st = steps[j - 1];
+        const bool shared = j == n;
+        // a single channel is an output of the layer below: masked on the way out; the shared
+        // pass completes the outputs of layer lo - 1
+        msd::PostMask pm{0, st.x};
+        if (shared) {
+            pm = msd::PostMask{st.g.C, {nullptr, 0, 0, 0, 0, 0}};
+            *masked = false;
+            if (lo - 1 >= 0) {
+                pm = msd::PostMask{(int)(c - a.widths[lo - 1]), x};
+                *masked = true;
+            }
+            st.g.reverse = msd::knob(msd::kKnobBlockSnake, 1) && !(pass_no & 1);
+        }
+        const int64_t region = partial_region_floats(a.ndim, st.g.C, j);
         msd::ReduceJob *job = nullptr;
         MSD_TRY(pending->next(fn, region, &job));
         ProfileScope scope(3, s);
-        g2.reverse = msd::knob(msd::kKnobBlockSnake, 1) && ((i >> 1) & 1);
-        const msd::LayerPair pair{d_lo, d_hi, w_hi, gk_hi};
-        const hipError_t e = msd::fast_backward_xkb_2d(g2, gy2, x, w_lo, gx, pm, gk_lo, (float *)gb_lower, (float *)ws, s,
-                                                       job, &pair);
+        const msd::LayerGroup *grp = j > 1 ? &st.group : nullptr;
+        const hipError_t e =
+            st.lean ? msd::fast_backward_one_channel_2d(st.g, st.gy, st.x, st.k, st.gx, pm, st.gk, (float *)ws, s, job,
+                                                        grp)
+                    : msd::fast_backward_xkb_2d(st.g, st.gy, st.x, st.k, st.gx, pm, st.gk,
+                                                shared ? (float *)gb_lowest : nullptr, (float *)ws, s, job, grp);
         if (e != hipSuccess) return hip_fail(fn, e);
         if (job) pending->taken(region);
     }
@@ -967,6 +1005,7 @@ int msd_block_backward(int dtype, int ndim, int64_t batch, int64_t c_in, int dep
         pending.capacity = (workspace_bytes - layer_ws) / (int64_t)sizeof(float);
     }
     bool masked = false;   // the mask of the current layer was already applied by the previous backward_x
+    int groups_done = 0;
     for (int i = depth - 1; i >= 0; i--) {
         const int64_t w = widths[i], first = last - w, b0 = b1 - w;
         const char *out_i = (const char *)stack + first * stack_strides[1] * a.elem;
@@ -981,16 +1020,24 @@ int msd_block_backward(int dtype, int ndim, int64_t batch, int64_t c_in, int dep
                                            grads_strides, stream));
         masked = false;
         void *gb = grad_bias ? (char *)grad_bias + b0 * a.elem : nullptr;
-        if (pair_candidate(a, i, need_input_grad != 0)) {
-            // this layer and the one below it in two launches that move every shared channel once
+        {
+            // this layer and the one or two below it in launches that move every shared channel once
+            int sizes[2];
+            const int tries = group_sizes(a, i, first, need_input_grad != 0, sizes);
             bool done = false;
-            MSD_TRY(block_pair_fused(fn, a, i, first, stack, stack_strides, grads, grads_strides, weights, grad_weights,
-                                     grad_bias ? (char *)grad_bias + (b0 - 1) * a.elem : nullptr, workspace,
-                                     workspace_bytes, (hipStream_t)stream, &pending, &masked, &done));
+            int n = 0;
+            for (int t = 0; t < tries && !done; t++) {
+                n = sizes[t];
+                MSD_TRY(block_group_fused(fn, a, i, n, first, stack, stack_strides, grads, grads_strides, weights,
+                                          grad_weights, grad_bias ? (char *)grad_bias + (b0 - (n - 1)) * a.elem : nullptr,
+                                          workspace, workspace_bytes, (hipStream_t)stream, &pending, groups_done,
+                                          &masked, &done));
+            }
             if (done) {
-                last = first - 1;
-                b1 = b0 - 1;
-                i--;
+                groups_done++;
+                last = first - (n - 1);
+                b1 = b0 - (n - 1);
+                i -= n - 1;
                 continue;
             }
         }

@@ -1,9 +1,10 @@
-// Backward pass of one layer over ONE input channel, 2D, fp32: grad_input of that channel,
-// the nine weight gradients of that channel, and the channel's ReLU mask on the way out.
+// Backward pass of one layer (or of two layers at once) over ONE input channel, 2D, fp32:
+// grad_input of that channel, the nine weight gradients of that channel per layer, and the
+// channel's ReLU mask on the way out.
 //
-// The dense block's backward loop takes its layers two at a time (msd_api.hip): the upper
-// layer of a pair first has to finish the gradient of the channel the lower layer wrote, one
-// channel out of up to a hundred.  The fused kernel (msd_bwdxk_impl.h) does that too, but its
+// The dense block's backward loop takes its layers two or three at a time (msd_api.hip): the
+// upper layers of such a group first have to finish the gradients of the channels the lower
+// layers wrote, one channel at a time out of up to a hundred.  The fused kernel (msd_bwdxk_impl.h) does that too, but its
 // pipeline of 16-channel blocks on the matrix cores runs in full for the one channel (20 us at
 // 1024 x 1024); here the channel is four planes of memory traffic and 18 multiply-adds per
 // voxel on the vector pipe: the gather of msd_rows.h (the same one, so the same values), one
@@ -26,31 +27,35 @@ struct Args {
     RowTeams rt;
     int ngroups, total_groups, tiles_per_wg;
     int masked;
-    int gy_sb, gy_sy, x_sb, x_sy, gx_sb, gx_sy;
+    int gy_sb, gy_sc, gy_sy, x_sb, x_sy, gx_sb, gx_sy;
+    UpperDilations up;   // the second layer's dilation where it has its own
 };
 
-template <int V>
+// WOUT layers (output gradients in consecutive channels of gy, weights kw and kw1).
+template <int V, int WOUT>
 __global__ __launch_bounds__(kThreads) void bwd_one_channel(const Args a, const float *__restrict__ gyp,
                                                             const float *__restrict__ xp, float *__restrict__ gxp,
                                                             const float *__restrict__ actp,
-                                                            const float *__restrict__ kw, float *__restrict__ part)
+                                                            const float *__restrict__ kw,
+                                                            const float *__restrict__ kw1, float *__restrict__ part)
 {
     extern __shared__ float lds[];
+    constexpr int KR = WOUT * K;
     const Geom &g = a.g;
     const RowTeams &rt = a.rt;
     const int tid = threadIdx.x;
     const int team = tid / rt.lpr, lane = tid % rt.lpr;
-    float *S = lds + (size_t)team * NPQ * V * rt.lpr;
-    float w[K];
+    float *S = lds + (size_t)team * WOUT * NPQ * V * rt.lpr;
+    float w[KR];
 #pragma unroll
-    for (int t = 0; t < K; t++) w[t] = kw[t];     // uniform: scalar loads
-    float ksum[K];
+    for (int t = 0; t < KR; t++) w[t] = t < K ? kw[t] : kw1[t - K];     // uniform: scalar loads
+    float ksum[KR];
 #pragma unroll
-    for (int t = 0; t < K; t++) ksum[t] = 0.f;
+    for (int t = 0; t < KR; t++) ksum[t] = 0.f;
     const int x0 = lane * V;
     const int xc = min(x0, g.W - V);
     const View<const float> none{nullptr, 0, 0, 0, 0, 0};
-    const View<const float> gyv{gyp, a.gy_sb, 0, 0, a.gy_sy, 1};
+    const View<const float> gyv{gyp, a.gy_sb, a.gy_sc, 0, a.gy_sy, 1};
 
     for (int ti = 0; ti < a.tiles_per_wg; ti++) {
         const int grp = blockIdx.x + ti * gridDim.x;          // uniform
@@ -67,27 +72,29 @@ __global__ __launch_bounds__(kThreads) void bwd_one_channel(const Args a, const 
         load_vec<V>(xp + xo, xv);
         load_vec<V>(gxp + go, gv);
         if (a.masked) load_vec<V>(actp + go, m);   // uniform; the activations share grad_input's layout
-        float own[1][NPQ][V];
-        stage_source_rows<2, false, 1, V>(g, rt, none, gyv, b, 0, y, lane, act, S, own);
-        float tv[K][V];
+        float own[WOUT][NPQ][V];
+        stage_source_rows<2, false, WOUT, V>(g, rt, none, gyv, b, 0, y, lane, act, S, own, a.up);
+        float tv[KR][V];
 #pragma unroll
-        for (int i = 0; i < V; i++) {
-            const SideTaps<V> side(min(x0 + i, g.W - 1), g.W, g.dil, rt.lpr);
+        for (int i = 0; i < V; i++)
 #pragma unroll
-            for (int pq = 0; pq < NPQ; pq++) {
-                float t0, t2;
-                side.read(S + (size_t)pq * V * rt.lpr, t0, t2);
-                tv[pq * 3 + 0][i] = t0;
-                tv[pq * 3 + 1][i] = own[0][pq][i];
-                tv[pq * 3 + 2][i] = t2;
+            for (int co = 0; co < WOUT; co++) {
+                const SideTaps<V> side(min(x0 + i, g.W - 1), g.W, dilation_of(g, a.up, co), rt.lpr);
+#pragma unroll
+                for (int pq = 0; pq < NPQ; pq++) {
+                    float t0, t2;
+                    side.read(S + (size_t)(co * NPQ + pq) * V * rt.lpr, t0, t2);
+                    tv[co * K + pq * 3 + 0][i] = t0;
+                    tv[co * K + pq * 3 + 1][i] = own[co][pq][i];
+                    tv[co * K + pq * 3 + 2][i] = t2;
+                }
             }
-        }
         __syncthreads();                          // the staged rows may be overwritten from here on
 #pragma unroll
         for (int i = 0; i < V; i++) {
             float sum = w[0] * tv[0][i];
 #pragma unroll
-            for (int t = 1; t < K; t++) sum += w[t] * tv[t][i];
+            for (int t = 1; t < KR; t++) sum += w[t] * tv[t][i];
             gv[i] += sum;
             if (a.masked) gv[i] = 0.f < m[i] ? gv[i] : 0.f;
         }
@@ -96,7 +103,7 @@ __global__ __launch_bounds__(kThreads) void bwd_one_channel(const Args a, const 
 #pragma unroll
         for (int i = 0; i < V; i++) xv[i] = act ? xv[i] : 0.f;
 #pragma unroll
-        for (int t = 0; t < K; t++)
+        for (int t = 0; t < KR; t++)
 #pragma unroll
             for (int i = 0; i < V; i++) ksum[t] += tv[t][i] * xv[i];
     }
@@ -105,16 +112,16 @@ __global__ __launch_bounds__(kThreads) void bwd_one_channel(const Args a, const 
     __syncthreads();
     const int wave = tid / kWave, wl = tid % kWave, nwaves = blockDim.x / kWave;
 #pragma unroll
-    for (int t = 0; t < K; t++) {
+    for (int t = 0; t < KR; t++) {
         float s = ksum[t];
 #pragma unroll
         for (int off = kWave / 2; off > 0; off >>= 1) s += __shfl_down(s, off, kWave);
-        if (wl == 0) lds[wave * K + t] = s;
+        if (wl == 0) lds[wave * KR + t] = s;
     }
     __syncthreads();
-    if (tid < K) {
+    if (tid < KR) {                               // column = layer * 9 + tap
         float s = 0.f;
-        for (int v = 0; v < nwaves; v++) s += lds[v * K + tid];
+        for (int v = 0; v < nwaves; v++) s += lds[v * KR + tid];
         part[(int64_t)tid * kMaxPartialRows + blockIdx.x] = s;
     }
 }
@@ -136,7 +143,7 @@ int choose_vec(const Geom &g, const View<const float> &gy, const View<const floa
 bool in_range(const Geom &g, const View<const float> &v)
 {
     const int64_t lim = (int64_t)1 << 31;
-    return v.sx == 1 && v.sb < lim && v.sy < lim && (int64_t)(g.H - 1) * v.sy + g.W < lim;
+    return v.sx == 1 && v.sb < lim && v.sc < lim && v.sy < lim && (int64_t)(g.H - 1) * v.sy + g.W < lim;
 }
 
 }  // namespace bwd1
@@ -144,19 +151,39 @@ bool in_range(const Geom &g, const View<const float> &v)
 bool fast_backward_one_channel_supported_2d(const Geom &g, const View<const float> &gy, const View<const float> &x,
                                             const View<float> &gx)
 {
-    if (g.ndim != 2 || g.C != 1 || g.Wd != 1 || g.D != 1) return false;
+    if (g.ndim != 2 || g.C != 1 || (g.Wd != 1 && g.Wd != 2) || g.D != 1) return false;
     const View<const float> gxc{gx.p, gx.sb, gx.sc, gx.sz, gx.sy, gx.sx};
     if (!bwd1::in_range(g, gy) || !bwd1::in_range(g, x) || !bwd1::in_range(g, gxc)) return false;
     RowTeams rt;
     return bwd1::choose_vec(g, gy, x, gx, &rt) != 0;
 }
 
+template <int WOUT>
+static void launch_one_channel(int v, dim3 grid, dim3 block, size_t lds, hipStream_t s, const bwd1::Args &a,
+                               const float *gy, const float *x, float *gx, const float *act, const float *k,
+                               const float *k1, float *part)
+{
+    if (v == 4)
+        hipLaunchKernelGGL((bwd1::bwd_one_channel<4, WOUT>), grid, block, lds, s, a, gy, x, gx, act, k, k1, part);
+    else if (v == 2)
+        hipLaunchKernelGGL((bwd1::bwd_one_channel<2, WOUT>), grid, block, lds, s, a, gy, x, gx, act, k, k1, part);
+    else
+        hipLaunchKernelGGL((bwd1::bwd_one_channel<1, WOUT>), grid, block, lds, s, a, gy, x, gx, act, k, k1, part);
+}
+
 hipError_t fast_backward_one_channel_2d(const Geom &g, const View<const float> &gy, const View<const float> &x,
                                         const float *k, const View<float> &gx, const PostMask &pm, float *gk,
-                                        float *ws, hipStream_t s, ReduceJob *defer)
+                                        float *ws, hipStream_t s, ReduceJob *defer, const LayerGroup *group)
 {
+    if (g.Wd != 1 && g.Wd != 2) return hipErrorInvalidValue;
+    if (group && (group->n != 2 || g.Wd != 2)) return hipErrorInvalidValue;
     bwd1::Args a;
     a.g = g;
+    a.up = UpperDilations{{0, 0}};
+    if (group) {
+        a.g.dil = group->dil[0];
+        a.up.d[0] = group->dil[1];
+    }
     const int v = bwd1::choose_vec(g, gy, x, gx, &a.rt);
     if (v == 0) return hipErrorInvalidConfiguration;
     a.ngroups = (g.H + a.rt.rpw - 1) / a.rt.rpw;
@@ -166,28 +193,29 @@ hipError_t fast_backward_one_channel_2d(const Geom &g, const View<const float> &
     const int wgs = (int)std::min<int64_t>(total, kMaxPartialRows);
     a.tiles_per_wg = (int)((total + wgs - 1) / wgs);
     a.masked = pm.from < g.C;
-    a.gy_sb = (int)gy.sb; a.gy_sy = (int)gy.sy;
+    a.gy_sb = (int)gy.sb; a.gy_sc = (int)gy.sc; a.gy_sy = (int)gy.sy;
     a.x_sb = (int)x.sb; a.x_sy = (int)x.sy;
     a.gx_sb = (int)gx.sb; a.gx_sy = (int)gx.sy;
     const float *actp = a.masked ? pm.act.p : x.p;
     float *part = defer ? const_cast<float *>(defer->part) : ws + backward_k_mask_floats(g);
-    const size_t lds = std::max((size_t)a.rt.rpw * bwd1::NPQ * v * a.rt.lpr, (size_t)(bwd1::kThreads / kWave) * bwd1::K) *
-                       sizeof(float);
+    const size_t lds = std::max((size_t)a.rt.rpw * g.Wd * bwd1::NPQ * v * a.rt.lpr,
+                                (size_t)(bwd1::kThreads / kWave) * g.Wd * bwd1::K) * sizeof(float);
     const dim3 grid(wgs), block(a.rt.lpr * a.rt.rpw);
-    if (v == 4)
-        hipLaunchKernelGGL(bwd1::bwd_one_channel<4>, grid, block, lds, s, a, gy.p, x.p, gx.p, actp, k, part);
-    else if (v == 2)
-        hipLaunchKernelGGL(bwd1::bwd_one_channel<2>, grid, block, lds, s, a, gy.p, x.p, gx.p, actp, k, part);
+    // the second layer's weights follow the first's, or are another layer's
+    const float *k1 = group ? group->k_up[0] : k + bwd1::K;
+    if (g.Wd == 2)
+        launch_one_channel<2>(v, grid, block, lds, s, a, gy.p, x.p, gx.p, actp, k, k1, part);
     else
-        hipLaunchKernelGGL(bwd1::bwd_one_channel<1>, grid, block, lds, s, a, gy.p, x.p, gx.p, actp, k, part);
+        launch_one_channel<1>(v, grid, block, lds, s, a, gy.p, x.p, gx.p, actp, k, k1, part);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    const int64_t nk = bwd1::K;
+    const int64_t nk = (int64_t)g.Wd * bwd1::K;
+    const ReduceJob job{part, gk, nullptr, nk, nk, wgs, {group ? group->gk_up[0] : nullptr, nullptr},
+                        group ? (int64_t)bwd1::K : nk};
     if (defer) {
-        *defer = ReduceJob{part, gk, nullptr, nk, nk, wgs, nullptr, nk};
+        *defer = job;
         return hipSuccess;
     }
-    const ReduceJob job{part, gk, nullptr, nk, nk, wgs, nullptr, nk};
     return reduce_columns_batch(&job, 1, s);
 }
 

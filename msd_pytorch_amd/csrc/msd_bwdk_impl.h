@@ -296,11 +296,9 @@ __global__ __launch_bounds__(kThreads, 2) void bwdk_mfma(Geom g, int remap, int 
 // l, l + 64, ... in order, then the 64 lane sums are added by a fixed shuffle
 // tree, so the result does not depend on scheduling.  Columns [0, nk) go to the
 // weight gradient, the following ones to the bias gradient; both accumulate.
-// Columns [split, nk) go to gk1 instead (the weight gradient of a second layer) where split < nk.
 static __global__ __launch_bounds__(256) void reduce_columns(const float *__restrict__ part, int rows, int64_t nk,
                                                              int64_t ncols, float *__restrict__ gk,
-                                                             float *__restrict__ gb, float *__restrict__ gk1,
-                                                             int64_t split)
+                                                             float *__restrict__ gb)
 {
     const int64_t col = (int64_t)blockIdx.x * (256 / kWave) + threadIdx.x / kWave;
     if (col >= ncols) return;
@@ -312,10 +310,7 @@ static __global__ __launch_bounds__(256) void reduce_columns(const float *__rest
     for (int off = kWave / 2; off > 0; off >>= 1) s += __shfl_down(s, off, kWave);
     if (l == 0) {
         if (col < nk) {
-            if (col < split)
-                gk[col] += s;
-            else
-                gk1[col - split] += s;
+            gk[col] += s;
         } else {
             gb[col - nk] += s;
         }
@@ -559,8 +554,7 @@ hipError_t launch_rows(const Geom &g, const View<const float> &out, const View<c
     if (e != hipSuccess) return e;
     const int64_t nk = (int64_t)g.Wd * g.C * K;
     const int64_t ncols = nk + (want_bias ? g.Wd : 0);
-    hipLaunchKernelGGL(reduce_columns, dim3((ncols + 3) / 4), dim3(256), 0, s, part, rows, nk, ncols, gk, gb,
-                       (float *)nullptr, nk);
+    hipLaunchKernelGGL(reduce_columns, dim3((ncols + 3) / 4), dim3(256), 0, s, part, rows, nk, ncols, gk, gb);
     return hipGetLastError();
 }
 
@@ -641,8 +635,7 @@ hipError_t launch(const Geom &g, bool relu, const View<const float> &out, const 
     if (e != hipSuccess) return e;
     const int64_t nk = (int64_t)g.Wd * g.C * K;
     const int64_t ncols = nk + (want_bias ? g.Wd : 0);
-    hipLaunchKernelGGL(reduce_columns, dim3((ncols + 3) / 4), dim3(256), 0, s, part, rows, nk, ncols, gk, gb,
-                       (float *)nullptr, nk);
+    hipLaunchKernelGGL(reduce_columns, dim3((ncols + 3) / 4), dim3(256), 0, s, part, rows, nk, ncols, gk, gb);
     return hipGetLastError();
 }
 

@@ -5,9 +5,9 @@ namespace msd {
 
 hipError_t fast_backward_xkb_2d_long(const Geom &g, const View<const float> &gy, const View<const float> &x,
                                      const float *k, const View<float> &gx, const PostMask &pm, float *gk, float *gb,
-                                     float *ws, hipStream_t s, ReduceJob *defer, const LayerPair *pair)
+                                     float *ws, hipStream_t s, ReduceJob *defer, const LayerGroup *group)
 {
-    return bwdxk::xkb_nd<2, true>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
+    return bwdxk::xkb_nd<2, true>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, group);
 }
 
 }  // namespace msd

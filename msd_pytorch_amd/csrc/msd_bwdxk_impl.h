@@ -67,19 +67,19 @@ struct Args {
     RowTeams rt;
     int remap, tiles_per_wg, ngroups, total_groups;
     int group_step;      // 1: a workgroup walks consecutive row groups; > 1: every group_step-th one
-    Plane gy;            // masked output gradient, one or two channels
+    Plane gy;            // masked output gradient, one to three channels
     Plane x;             // input channels
     Plane gx;            // grad_input channels (written through a cast)
     int mask_from;       // activations (viewed like grad_input) mask the channels >= mask_from
     int want_bias;
     RowSegments sg;      // LONG instances
-    int dil1;            // two output channels: the dilation of the second one's taps (two layers in one pass)
+    UpperDilations up;   // layers of a dense block in one pass: the dilations of output channels 1 and 2
 };
 
 // The waves' tiles share the LDS of the staged rows (two outputs at four voxels per lane: the
 // tiles alone are 79 KB).
 template <int NDIM, int V, int WOUT>
-constexpr bool tiles_over_staging() { return NDIM == 2 && V == 4 && WOUT == 2; }
+constexpr bool tiles_over_staging() { return NDIM == 2 && ((V == 4 && WOUT == 2) || WOUT == 3); }
 
 // Workgroups (of four waves) that are resident per CU.  The 3D kernel with one voxel per lane
 // (pipeline stages of 16 voxels, arguments read again per tile, row arithmetic on the scalar
@@ -115,7 +115,7 @@ template <int NDIM, int V, int NCB, int WOUT, bool LONG, bool BIG = LONG>
 __global__ __launch_bounds__(kThreads, (resident_per_cu<NDIM, V, NCB, WOUT, LONG>()))
 void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *__restrict__ xp,
                     float *__restrict__ gxp, const float *__restrict__ actp, const float *__restrict__ kw,
-                    const float *__restrict__ kw1, float *__restrict__ part)
+                    const float *__restrict__ kw1, const float *__restrict__ kw2, float *__restrict__ part)
 {
     // the pointers are separate arguments so that they can carry __restrict__: the weights
     // are then known not to change under the stores to grad_input and stay scalar loads
@@ -326,17 +326,17 @@ void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *_
             float own[WOUT][NPQ][V];
             if (segmented) {
                 if constexpr (SEG)
-                    stage_source_segment<NDIM, WOUT, V>(g, rt, a.sg, gyv, b, zc, yc, xs, lane, rowok, S, own, a.dil1);
+                    stage_source_segment<NDIM, WOUT, V>(g, rt, a.sg, gyv, b, zc, yc, xs, lane, rowok, S, own, a.up);
             } else {
-                stage_source_rows<NDIM, false, WOUT, V>(g, rt, none, gyv, b, zc, yc, lane, act, S, own, a.dil1);
+                stage_source_rows<NDIM, false, WOUT, V>(g, rt, none, gyv, b, zc, yc, lane, act, S, own, a.up);
             }
             // per voxel: all LDS reads first, so that their latencies overlap, then the sums
 #pragma unroll
             for (int i = 0; i < V; i++)
 #pragma unroll
                 for (int co = 0; co < WOUT; co++) {
-                    // (the second output channel may have a dilation of its own, and with it its own x-taps)
-                    const int dil = (WOUT > 1 && co > 0 && a.dil1 > 0) ? a.dil1 : g.dil;
+                    // (the upper output channels may have dilations of their own, and with them their own x-taps)
+                    const int dil = dilation_of(g, a.up, co);
                     const SideTaps<V> side = segmented ? SideTaps<V>(x0 + i, g.W, dil, rt.lpr, xs, V * rt.lpr)
                                                        : SideTaps<V>(min(x0 + i, g.W - 1), g.W, dil, rt.lpr);
                     float ra[NPQ][4];
@@ -421,7 +421,7 @@ void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *_
         auto load_weights = [&](int ci, float (&w)[KR]) {
 #pragma unroll
             for (int co = 0; co < WOUT; co++) {
-                const float *kc = (co == 0 ? kw : kw1) + (uint32_t)(ci * K);
+                const float *kc = (co == 0 ? kw : (co == 1 ? kw1 : kw2)) + (uint32_t)(ci * K);
 #pragma unroll
                 for (int t = 0; t < K; t++) w[co * K + t] = kc[t];
             }
@@ -684,7 +684,7 @@ bool fits(const Geom &g, int V, const View<const float> &gy, const View<const fl
     const size_t kr = (size_t)g.Wd * Taps<NDIM>::K + 1;
     const size_t staged = (size_t)rt.rpw * g.Wd * RowTaps<NDIM>::NPQ * (V * rt.lpr + sg.halo) * 4;
     const size_t tiles = (size_t)kWaves * kr * (kWave * V + 4) * 4;
-    const bool over = NDIM == 2 && V == 4 && g.Wd == 2;   // tiles_over_staging()
+    const bool over = NDIM == 2 && ((V == 4 && g.Wd == 2) || g.Wd == 3);   // tiles_over_staging()
     if ((over ? std::max(staged, tiles) : staged + tiles) > (over ? kMaxLdsBytesAsked : kMaxLdsBytes)) return false;
     return rows_aligned(gy, g.W, V) && rows_aligned(gx, g.W, V);
 }
@@ -702,21 +702,21 @@ int choose_vec(const Geom &g, int vmax, const View<const float> &gy, const View<
     return 0;
 }
 
-// `pair`: the two output channels are two layers of a dense block (g.dil is then the larger of
-// their dilations, which is what the row segments' halo is sized for).
+// `group`: the output channels are layers of a dense block (g.dil is then the largest of their
+// dilations, which is what the row segments' halo is sized for).
 template <int NDIM, int V, int NCB, int WOUT, bool LONG, bool BIG = LONG>
 hipError_t launch(const Geom &g, const View<const float> &gy, const View<const float> &x, const float *k,
                   const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws, hipStream_t s,
-                  ReduceJob *defer, const LayerPair *pair)
+                  ReduceJob *defer, const LayerGroup *group)
 {
     constexpr int K = Taps<NDIM>::K;
     Args a;
     a.g = g;
-    a.dil1 = 0;
-    if (pair) {
-        if (WOUT != 2) return hipErrorInvalidValue;
-        a.g.dil = pair->dil0;
-        a.dil1 = pair->dil1;
+    a.up = UpperDilations{{0, 0}};
+    if (group) {
+        if (WOUT != group->n || WOUT < 2 || WOUT > kMaxLayerGroup) return hipErrorInvalidValue;
+        a.g.dil = group->dil[0];
+        for (int co = 1; co < WOUT; co++) a.up.d[co - 1] = group->dil[co];
     }
     a.sg = RowSegments{1, 0};
     make_row_teams(g, V, &a.rt, LONG ? &a.sg : nullptr);
@@ -755,36 +755,44 @@ hipError_t launch(const Geom &g, const View<const float> &gy, const View<const f
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLdsBytesAsked);
         if (e != hipSuccess) return e;
     }
-    // the weights of the second output channel follow those of the first, or are another layer's
-    const float *k1 = pair ? pair->k1 : k + (int64_t)g.C * K;
+    // the weights of the upper output channels follow those of the first, or are other layers'
+    const float *k1 = group ? group->k_up[0] : k + (int64_t)g.C * K;
+    const float *k2 = group ? group->k_up[1] : k + (int64_t)2 * g.C * K;
     hipLaunchKernelGGL((bwd_rows_fused<NDIM, V, NCB, WOUT, LONG, BIG>), dim3(rows, 1, chunks), dim3(a.rt.lpr * a.rt.rpw), lds, s, a,
-                       gy.p, x.p, gx.p, actp, k, k1, part);
+                       gy.p, x.p, gx.p, actp, k, k1, k2, part);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     const int64_t nk = (int64_t)WOUT * g.C * K;
     const int64_t ncols = nk + (a.want_bias ? WOUT : 0);
-    // columns [0, split) of the partial sums go to gk, [split, nk) to gk1
-    const int64_t split = pair ? (int64_t)g.C * K : nk;
-    float *gk1 = pair ? pair->gk1 : nullptr;
+    // a group's columns: [0, split) of the partial sums go to gk, the next `split` ones to the
+    // second layer's weight gradient, the rest to the third's
+    const ReduceJob job{part, gk, gb, nk, ncols, rows, {group ? group->gk_up[0] : nullptr, group ? group->gk_up[1] : nullptr},
+                        group ? (int64_t)g.C * K : nk};
     if (defer) {
-        *defer = ReduceJob{part, gk, gb, nk, ncols, rows, gk1, split};
+        *defer = job;
         return hipSuccess;
     }
-    hipLaunchKernelGGL(bwdk::reduce_columns, dim3((ncols + 3) / 4), dim3(256), 0, s, part, rows, nk, ncols, gk, gb, gk1,
-                       split);
+    if (group) return reduce_columns_batch(&job, 1, s);   // (adds in the same order)
+    hipLaunchKernelGGL(bwdk::reduce_columns, dim3((ncols + 3) / 4), dim3(256), 0, s, part, rows, nk, ncols, gk, gb);
     return hipGetLastError();
 }
 
 template <int NDIM, int V, int WOUT, bool LONG, bool BIG = LONG>
 hipError_t pick_ncb(const Geom &g, const View<const float> &gy, const View<const float> &x, const float *k,
                     const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws, hipStream_t s,
-                    ReduceJob *defer, const LayerPair *pair)
+                    ReduceJob *defer, const LayerGroup *group)
 {
     const int need = (g.C + kChanBlock - 1) / kChanBlock;
-    if (need <= 1) return launch<NDIM, V, 1, WOUT, LONG, BIG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
-    if (need <= 2) return launch<NDIM, V, 2, WOUT, LONG, BIG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
-    if (need <= 4) return launch<NDIM, V, 4, WOUT, LONG, BIG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
-    return launch<NDIM, V, 8, WOUT, LONG, BIG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
+    if (need <= 1) return launch<NDIM, V, 1, WOUT, LONG, BIG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, group);
+    if (need <= 2) return launch<NDIM, V, 2, WOUT, LONG, BIG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, group);
+    // (three output channels: more than 64 channels per chunk do not fit the registers; the
+    // channels then go in chunks of 64 over the grid's third dimension)
+    if constexpr (WOUT >= 3) {
+        return launch<NDIM, V, 4, WOUT, LONG, BIG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, group);
+    } else {
+        if (need <= 4) return launch<NDIM, V, 4, WOUT, LONG, BIG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, group);
+        return launch<NDIM, V, 8, WOUT, LONG, BIG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, group);
+    }
 }
 
 // Widest vector for two output channels (2D only): twice the gathered values per voxel must
@@ -809,11 +817,19 @@ enum Mode { kUnsupported = 0, kPlain = 1, kLong = 2 };
 template <int NDIM>
 Mode xkb_mode(const Geom &g, const View<const float> &gy, const View<const float> &x, const View<float> &gx)
 {
-    if (g.Wd != 1 && !(NDIM == 2 && g.Wd == 2)) return kUnsupported;
+    if (g.Wd != 1 && !(NDIM == 2 && (g.Wd == 2 || g.Wd == 3))) return kUnsupported;
     if (x.sx != 1 || gy.sx != 1 || gx.sx != 1) return kUnsupported;
     if (!small_strides(g, gy) || !small_strides(g, x) || !small_strides(g, gx)) return kUnsupported;
-    const int vmax = g.Wd == 2 ? kMaxVecTwoOutputs : 4;
+    const int vmax = g.Wd >= 2 ? kMaxVecTwoOutputs : 4;
     const View<const float> gxc{gx.p, gx.sb, gx.sc, gx.sz, gx.sy, gx.sx};
+    if (g.Wd == 3) {
+        // three output channels: aligned rows of whole groups of four voxels, two voxels per lane,
+        // offsets within 32 bits; nothing else
+        if (!x_offsets_fit(g, x, false) || !x_offsets_fit(g, gxc, false)) return kUnsupported;
+        if (g.W % 4 == 0 && rows_aligned(x, g.W, 4) && choose_vec<NDIM>(g, kMaxVecTwoOutputs, gy, x, gx, true) == 2)
+            return kLong;
+        return kUnsupported;
+    }
     const int vmax_plain = g.Wd == 2 ? kMaxVecTwoOutputsPlain : 4;
     if (x_offsets_fit(g, x, false) && x_offsets_fit(g, gxc, false) &&
         choose_vec<NDIM>(g, vmax_plain, gy, x, gx, false) != 0)
@@ -826,7 +842,7 @@ Mode xkb_mode(const Geom &g, const View<const float> &gy, const View<const float
 template <int NDIM, bool LONG>
 hipError_t xkb_nd(const Geom &g, const View<const float> &gy, const View<const float> &x, const float *k,
                   const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws, hipStream_t s,
-                  ReduceJob *defer, const LayerPair *pair = nullptr)
+                  ReduceJob *defer, const LayerGroup *group = nullptr)
 {
     // 3D: one voxel per lane keeps the 27 gathered values per voxel and the pipeline buffers in registers
     int vmax = knob(NDIM == 3 ? kKnobBwdkVec3d : kKnobBwdkVec2d, NDIM == 3 ? 1 : 4);
@@ -836,7 +852,7 @@ hipError_t xkb_nd(const Geom &g, const View<const float> &gy, const View<const f
         // wins, else the one with the most tiles (256 x 256, 100 channels: 58 -> 39 us).
         int best = 0;
         int64_t best_tiles = 0;
-        for (int v = g.Wd == 2 ? kMaxVecTwoOutputsPlain : 4; v >= 1; v /= 2) {
+        for (int v = g.Wd == 3 ? kMaxVecTwoOutputs : (g.Wd == 2 ? kMaxVecTwoOutputsPlain : 4); v >= 1; v /= 2) {
             RowTeams rt;
             if (!fits<NDIM>(g, v, gy, x, gx, LONG) || !make_row_teams(g, v, &rt)) continue;
             const int64_t tiles = (int64_t)g.B * ((rt.nrows + rt.rpw - 1) / rt.rpw);
@@ -848,6 +864,16 @@ hipError_t xkb_nd(const Geom &g, const View<const float> &gy, const View<const f
     int v = choose_vec<NDIM>(g, vmax, gy, x, gx, LONG);
     if (v == 0) v = choose_vec<NDIM>(g, 4, gy, x, gx, LONG);
     if constexpr (NDIM == 2) {
+        if (g.Wd == 3) {
+            // three output channels: two voxels per lane in the instance that cuts long rows into
+            // segments and is otherwise like the plain one (xkb_mode), also for rows that one
+            // workgroup covers (the plain form of it would spill registers)
+            if constexpr (LONG) {
+                if (choose_vec<2>(g, kMaxVecTwoOutputs, gy, x, gx, true) == 2)
+                    return pick_ncb<2, 2, 3, true, false>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, group);
+            }
+            return hipErrorInvalidConfiguration;
+        }
         if (g.Wd == 2) {
             constexpr int vmax2 = LONG ? kMaxVecTwoOutputs : kMaxVecTwoOutputsPlain;
             v = choose_vec<2>(g, std::min(vmax, vmax2), gy, x, gx, LONG);
@@ -859,16 +885,16 @@ hipError_t xkb_nd(const Geom &g, const View<const float> &gy, const View<const f
                 const bool segments_only = g.W % 4 == 0 && rows_aligned(x, g.W, 4) && x_offsets_fit(g, x, false) &&
                                            x_offsets_fit(g, gxc, false);
                 if (segments_only && vmax >= 4 && choose_vec<2>(g, 4, gy, x, gx, true) == 4)
-                    return pick_ncb<2, 4, 2, true, false>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
+                    return pick_ncb<2, 4, 2, true, false>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, group);
                 if (segments_only && v == 2)
-                    return pick_ncb<2, 2, 2, true, false>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
+                    return pick_ncb<2, 2, 2, true, false>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, group);
                 if (segments_only && v == 1)
-                    return pick_ncb<2, 1, 2, true, false>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
+                    return pick_ncb<2, 1, 2, true, false>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, group);
             }
             if constexpr (!LONG)
-                if (v == 4) return pick_ncb<2, 4, 2, false>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
-            if (v == 2) return pick_ncb<2, 2, 2, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
-            if (v == 1) return pick_ncb<2, 1, 2, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, pair);
+                if (v == 4) return pick_ncb<2, 4, 2, false>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, group);
+            if (v == 2) return pick_ncb<2, 2, 2, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, group);
+            if (v == 1) return pick_ncb<2, 1, 2, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, group);
             return hipErrorInvalidConfiguration;
         }
         if (v == 4) return pick_ncb<2, 4, 1, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, nullptr);

@@ -61,7 +61,7 @@ enum Knob {
     kKnobXcdRemap, kKnobBwdkVec2d, kKnobBwdkVec3d, kKnobBwdkBlocks,
     kKnobFwdVec2d, kKnobFwdVec3d, kKnobFwdSplit, kKnobFwdRows2d, kKnobBwdkRows, kKnobBlockFuse,
     kKnobBlockDefer, kKnobBwdkInterleave, kKnobBlockSnake, kKnobFwdClass3d, kKnobFwdLattice3d,
-    kKnobBlockPair,
+    kKnobBlockPair, kKnobBlockTriple,
     kKnobCount
 };
 int knob(Knob k, int dflt);
@@ -149,17 +149,21 @@ struct ReduceJob {
     float *gk, *gb;
     int64_t nk, ncols;
     int rows;
-    float *gk1;       // columns [split, nk) go here instead of to gk (a second layer's weight gradient)
-    int64_t split;    // nk where there is no second destination
+    float *gk_up[2];  // columns [split, 2 split) and [2 split, nk) go here instead of to gk (the weight
+                      // gradients of a second and a third layer)
+    int64_t split;    // nk where there is no other destination
 };
-// Two layers of a dense block as the two output channels of one fused backward pass over the
-// input channels they share: output channel 0 is the lower layer (dilation dil0, weights k,
-// weight gradient gk), output channel 1 the layer above it (dil1, k1, gk1; the first g.C of its
-// input channels).  The Geom's dilation is the larger of the two.
-struct LayerPair {
-    int dil0, dil1;
-    const float *k1;
-    float *gk1;
+// Two or three layers of a dense block as the output channels of one fused backward pass over
+// the input channels they share: output channel 0 is the lowest layer (dilation dil[0], the
+// call's weights k and weight gradient gk), output channel j the j-th layer above it (dil[j],
+// k_up[j - 1], gk_up[j - 1]; the first g.C of its input channels).  The Geom's dilation is the
+// largest of them.
+constexpr int kMaxLayerGroup = 3;
+struct LayerGroup {
+    int n;
+    int dil[kMaxLayerGroup];
+    const float *k_up[kMaxLayerGroup - 1];
+    float *gk_up[kMaxLayerGroup - 1];
 };
 constexpr int kReduceBatch = 16;
 // One launch for up to kReduceBatch pending reductions; every column is added in the same
@@ -176,7 +180,7 @@ bool fast_backward_xkb_supported_3d(const Geom &g, const View<const float> &gy, 
                                     const View<float> &gx);
 hipError_t fast_backward_xkb_2d(const Geom &g, const View<const float> &gy, const View<const float> &x, const float *k,
                                 const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws,
-                                hipStream_t s, ReduceJob *defer, const LayerPair *pair = nullptr);
+                                hipStream_t s, ReduceJob *defer, const LayerGroup *group = nullptr);
 hipError_t fast_backward_xkb_3d(const Geom &g, const View<const float> &gy, const View<const float> &x, const float *k,
                                 const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws,
                                 hipStream_t s, ReduceJob *defer);
@@ -184,18 +188,20 @@ hipError_t fast_backward_xkb_3d(const Geom &g, const View<const float> &gy, cons
 // not fit 32 bits; chosen by fast_backward_xkb_2d / _3d, not called directly
 hipError_t fast_backward_xkb_2d_long(const Geom &g, const View<const float> &gy, const View<const float> &x,
                                      const float *k, const View<float> &gx, const PostMask &pm, float *gk, float *gb,
-                                     float *ws, hipStream_t s, ReduceJob *defer, const LayerPair *pair = nullptr);
+                                     float *ws, hipStream_t s, ReduceJob *defer, const LayerGroup *group = nullptr);
 hipError_t fast_backward_xkb_3d_long(const Geom &g, const View<const float> &gy, const View<const float> &x,
                                      const float *k, const View<float> &gx, const PostMask &pm, float *gk, float *gb,
                                      float *ws, hipStream_t s, ReduceJob *defer);
 
-// One layer over one input channel (2D): grad_input, the channel's nine weight gradients, its
-// ReLU mask (pm.from == 0) on the way out.  msd_bwd1.hip.
+// One layer, or two (g.Wd output channels; `group`: two layers of a dense block), over one input
+// channel (2D): grad_input, the channel's nine weight gradients per layer, its ReLU mask
+// (pm.from == 0) on the way out.  msd_bwd1.hip.
 bool fast_backward_one_channel_supported_2d(const Geom &g, const View<const float> &gy, const View<const float> &x,
                                             const View<float> &gx);
 hipError_t fast_backward_one_channel_2d(const Geom &g, const View<const float> &gy, const View<const float> &x,
                                         const float *k, const View<float> &gx, const PostMask &pm, float *gk,
-                                        float *ws, hipStream_t s, ReduceJob *defer);
+                                        float *ws, hipStream_t s, ReduceJob *defer,
+                                        const LayerGroup *group = nullptr);
 
 inline bool fast_backward_xkb_supported(const Geom &g, const View<const float> &gy, const View<const float> &x,
                                         const View<float> &gx)

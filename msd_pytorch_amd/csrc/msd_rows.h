@@ -159,23 +159,33 @@ inline size_t staged_floats(const RowTeams &rt, int wout)
     return (size_t)wout * RowTaps<NDIM>::NPQ * rt.V * rt.lpr;
 }
 
+// Dilations of the output channels above the first where they have one of their own (two or
+// three layers of a dense block gathered in one pass); 0: the layer's dilation.
+struct UpperDilations {
+    int d[2];
+};
+__device__ __forceinline__ int dilation_of(const Geom &g, const UpperDilations &up, int co)
+{
+    return (co >= 1 && co <= 2 && up.d[co - 1] > 0) ? up.d[co - 1] : g.dil;
+}
+
 // Stage S[co][pq] of the team's row into LDS (see the header comment) and keep
 // the lane's own V values of every staged row in `own`.  Every lane of the
 // workgroup must call this; lanes outside the image (`act` false) stage zeros.
 // Ends with a workgroup barrier.
-// `dil1`: the dilation of the second output channel's taps where it has one of its own (two
-// layers of a dense block gathered in one pass); the layer's dilation otherwise.
+// `up`: the dilations of the output channels that have one of their own.
 template <int NDIM, bool RELU, int WOUT, int V>
 __device__ __forceinline__ void stage_source_rows(const Geom &g, const RowTeams &rt, const View<const float> &out,
                                                   const View<const float> &gy, int b, int z, int y, int lane,
                                                   bool act, float *__restrict__ S,
-                                                  float (&own)[WOUT][RowTaps<NDIM>::NPQ][V], int dil1 = 0)
+                                                  float (&own)[WOUT][RowTaps<NDIM>::NPQ][V],
+                                                  const UpperDilations up = UpperDilations{{0, 0}})
 {
     constexpr int NZ = Taps<NDIM>::NZ, NPQ = RowTaps<NDIM>::NPQ;
     const int x0 = min(lane * V, g.W - V);   // lanes past the row read a valid address; their values are dropped
 #pragma unroll
     for (int co = 0; co < WOUT; co++) {
-        const int dil = (WOUT > 1 && co > 0 && dil1 > 0) ? dil1 : g.dil;
+        const int dil = dilation_of(g, up, co);
         const AxisSources sz = NDIM == 3 ? adjoint_sources(z, g.D, dil) : single_source();
         const AxisSources sy = adjoint_sources(y, g.H, dil);
         // rows whose taps fold: within dil of a y (or z) border
@@ -238,7 +248,8 @@ template <int NDIM, int WOUT, int V>
 __device__ __forceinline__ void stage_source_segment(const Geom &g, const RowTeams &rt, const RowSegments &sg,
                                                      const View<const float> &gy, int b, int z, int y, int xs,
                                                      int lane, bool rowok, float *__restrict__ S,
-                                                     float (&own)[WOUT][RowTaps<NDIM>::NPQ][V], int dil1 = 0)
+                                                     float (&own)[WOUT][RowTaps<NDIM>::NPQ][V],
+                                                     const UpperDilations up = UpperDilations{{0, 0}})
 {
     constexpr int NZ = Taps<NDIM>::NZ, NPQ = RowTaps<NDIM>::NPQ;
     const int rs = V * rt.lpr + sg.halo;         // floats per staged row (the halo is sized for the larger dilation)
@@ -247,7 +258,7 @@ __device__ __forceinline__ void stage_source_segment(const Geom &g, const RowTea
     const int h = lane;                          // halo element of this lane, if any
 #pragma unroll
     for (int co = 0; co < WOUT; co++) {
-        const int dil = (WOUT > 1 && co > 0 && dil1 > 0) ? dil1 : g.dil;
+        const int dil = dilation_of(g, up, co);
         const AxisSources sz = NDIM == 3 ? adjoint_sources(z, g.D, dil) : single_source();
         const AxisSources sy = adjoint_sources(y, g.H, dil);
         const int hx = h < dil ? xs - dil + h : xs + V * rt.lpr + (h - dil);

@@ -149,6 +149,21 @@ INSTANCES = [
     ({"bwdk.vec2d": 4}, (1, 20, 2, (9, 512), 8)),
     ({"bwdk.vec2d": 4}, (2, 40, 2, (10, 256), 1)),
     ({"bwdk.vec2d": 4}, (1, 100, 2, (13, 256), 12)),
+    # three output channels in one fused pass (rows of whole groups of four voxels): rows that
+    # one workgroup covers (one to four rows each, lanes past the row's end) and rows in
+    # segments; one, two and four channel blocks per chunk, more than one chunk
+    ({}, (1, 9, 3, (7, 512), 3)),
+    ({}, (2, 20, 3, (9, 256), 8)),
+    ({}, (1, 40, 3, (5, 384), 2)),
+    ({}, (1, 100, 3, (6, 512), 5)),
+    ({}, (1, 9, 3, (7, 192), 3)),
+    ({}, (2, 40, 3, (5, 64), 2)),
+    ({}, (1, 70, 3, (6, 100), 5)),
+    ({}, (1, 9, 3, (7, 1024), 3)),
+    ({}, (2, 20, 3, (9, 1280), 8)),
+    ({}, (1, 40, 3, (5, 2048), 2)),
+    ({}, (1, 130, 3, (6, 1024), 5)),
+    ({}, (1, 20, 3, (7, 1026), 3)),                  # not covered by the fused kernel: two passes
 ]
 
 
@@ -169,7 +184,8 @@ def test_operators_under_a_forced_setting(cc, case):
 BLOCK_SETTINGS = [{"block.snake": 0}, {"block.snake": 1}, {"block.fuse": 0}, {"block.defer": 0},
                   {"xcd_remap": 0}, {"bwdk.interleave": 0}, {"fwd.class3d": 0}, {"fwd.lattice3d": 44},
                   {"block.pair": 0}, {"block.pair": 1}, {"block.pair": 1, "block.defer": 0},
-                  {"block.pair": 1, "block.snake": 0}]
+                  {"block.pair": 1, "block.snake": 0}, {"block.triple": 1}, {"block.triple": 0},
+                  {"block.triple": 1, "block.defer": 0}, {"block.triple": 1, "block.snake": 0}]
 
 
 @pytest.mark.parametrize("settings", BLOCK_SETTINGS, ids=lambda s: ",".join("%s=%d" % kv for kv in s.items()))
@@ -198,14 +214,21 @@ PAIR_BLOCKS = [
     ((33, 70), 2, 9, 2, [1, 2, 3, 4, 5, 6, 7, 8, 9]),
     ((20, 255), 1, 5, 1, [2, 7, 1, 4, 3]),          # odd rows: one voxel per lane in the one-channel step
     ((40, 64), 1, 20, 1, None),
+    ((10, 384), 1, 7, 1, [3, 1, 4, 1, 5, 9, 2]),    # two voxels per lane in the one-channel steps
+    ((8, 1280), 40, 6, 1, [2, 7, 1, 8, 2, 8]),      # three layers over more than 32 channels (the default's threshold)
+    ((6, 512), 70, 3, 2, [6, 1, 3]),                # three layers, channels in two chunks of the grid
 ]
 
+# "triples": three layers at a time wherever the kernels cover it (by default only where the
+# layers share at least 32 channels), two or one where they do not or where fewer are left
+GROUPINGS = {"triples": {"block.triple": 1}, "pairs": {"block.triple": 0}, "default": {}, "single": {"block.pair": 0}}
 
-@pytest.mark.parametrize("pair", [1, 0], ids=["paired", "single"])
+
+@pytest.mark.parametrize("grouping", list(GROUPINGS))
 @pytest.mark.parametrize("case", PAIR_BLOCKS, ids=lambda c: "x".join(map(str, c[0])) + "-d%d" % c[2])
-def test_block_backward_two_layers_at_a_time(case, pair):
+def test_block_backward_two_or_three_layers_at_a_time(case, grouping):
     size, c_in, depth, batch, dilations = case
-    with tuning({"block.pair": pair}):
+    with tuning(GROUPINGS[grouping]):
         check_block(2, size, c_in, 1, depth, batch, dilations=dilations, seed=11)
 
 
@@ -217,13 +240,13 @@ def test_paired_and_single_backward_agree_when_the_input_needs_no_gradient():
     from cases import rel_err
     x, dil, bias, ws, g = block_problem(2, (19, 384), 1, 1, 8, 2, seed=5)
     grads = {}
-    for pair in (0, 1):
-        with tuning({"block.pair": pair}):
+    for pair in (0, 1, 3):
+        with tuning({"block.pair": 0} if pair == 0 else {"block.triple": int(pair == 3)}):
             bd = bias.cuda().requires_grad_(True)
             wd = [w.cuda().requires_grad_(True) for w in ws]
             out = msd_block(x.cuda(), dil, bd, *wd)
             out.backward(g.cuda())
             torch.cuda.synchronize()
             grads[pair] = [bd.grad.clone()] + [w.grad.clone() for w in wd]
-    for a, b in zip(grads[0], grads[1]):
-        assert rel_err(a, b) <= 1e-5
+    for a, b, c in zip(grads[0], grads[1], grads[3]):
+        assert rel_err(a, b) <= 1e-5 and rel_err(a, c) <= 1e-5
