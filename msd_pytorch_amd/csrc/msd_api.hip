@@ -833,14 +833,14 @@ bool group_candidate(const BlockArgs &a, int i, int n, bool need_input_grad)
 }
 
 // Layers to take together from layer i down, most first.  Three where the shared pass is over
-// enough channels to gain from it (its tiles cost more to set up than a pair's), or wherever
-// possible when asked for ("block.triple" 1; 0: never).
+// enough channels to gain from it (its tiles cost more to set up than a pair's): 32, or the
+// value of "block.triple" (1: wherever possible; 0: never).
 int group_sizes(const BlockArgs &a, int i, int64_t first, bool need_input_grad, int (&sizes)[2])
 {
     int m = 0;
     const int triple = msd::knob(msd::kKnobBlockTriple, -1);
-    constexpr int64_t kTripleFromChannels = 32;
-    if (triple != 0 && group_candidate(a, i, 3, need_input_grad) && (triple > 0 || first - 2 >= kTripleFromChannels))
+    const int64_t from_channels = triple < 0 ? 32 : triple;
+    if (triple != 0 && group_candidate(a, i, 3, need_input_grad) && first - 2 >= from_channels)
         sizes[m++] = 3;
     if (group_candidate(a, i, 2, need_input_grad)) sizes[m++] = 2;
     return m;

@@ -33,7 +33,7 @@ struct Args {
 
 // WOUT layers (output gradients in consecutive channels of gy, weights kw and kw1).
 template <int V, int WOUT>
-__global__ __launch_bounds__(kThreads) void bwd_one_channel(const Args a, const float *__restrict__ gyp,
+__global__ __launch_bounds__(kThreads, 4) void bwd_one_channel(const Args a, const float *__restrict__ gyp,
                                                             const float *__restrict__ xp, float *__restrict__ gxp,
                                                             const float *__restrict__ actp,
                                                             const float *__restrict__ kw,
@@ -44,22 +44,27 @@ __global__ __launch_bounds__(kThreads) void bwd_one_channel(const Args a, const 
     const Geom &g = a.g;
     const RowTeams &rt = a.rt;
     const int tid = threadIdx.x;
-    const int team = tid / rt.lpr, lane = tid % rt.lpr;
-    float *S = lds + (size_t)team * WOUT * NPQ * V * rt.lpr;
+    const int team = tid / rt.lpr, lane0 = tid % rt.lpr;
     float w[KR];
 #pragma unroll
     for (int t = 0; t < KR; t++) w[t] = t < K ? kw[t] : kw1[t - K];     // uniform: scalar loads
     float ksum[KR];
 #pragma unroll
     for (int t = 0; t < KR; t++) ksum[t] = 0.f;
-    const int x0 = lane * V;
-    const int xc = min(x0, g.W - V);
     const View<const float> none{nullptr, 0, 0, 0, 0, 0};
     const View<const float> gyv{gyp, a.gy_sb, a.gy_sc, 0, a.gy_sy, 1};
 
     for (int ti = 0; ti < a.tiles_per_wg; ti++) {
         const int grp = blockIdx.x + ti * gridDim.x;          // uniform
         if (grp >= a.total_groups) break;
+        // what depends on the lane only is computed per tile on purpose (the lane number passes
+        // through an empty asm): hoisted out of the loop, the LDS positions of all the taps
+        // would occupy a hundred registers for a loop that mostly runs once
+        int lane = lane0;
+        asm volatile("" : "+v"(lane));
+        float *S = lds + (size_t)team * WOUT * NPQ * V * rt.lpr;
+        const int x0 = lane * V;
+        const int xc = min(x0, g.W - V);
         const int gi = grp % a.ngroups, b = grp / a.ngroups;
         const int row = gi * rt.rpw + team;
         const bool rowok = row < g.H;
@@ -74,42 +79,49 @@ __global__ __launch_bounds__(kThreads) void bwd_one_channel(const Args a, const 
         if (a.masked) load_vec<V>(actp + go, m);   // uniform; the activations share grad_input's layout
         float own[WOUT][NPQ][V];
         stage_source_rows<2, false, WOUT, V>(g, rt, none, gyv, b, 0, y, lane, act, S, own, a.up);
-        float tv[KR][V];
-#pragma unroll
-        for (int i = 0; i < V; i++)
-#pragma unroll
-            for (int co = 0; co < WOUT; co++) {
-                const SideTaps<V> side(min(x0 + i, g.W - 1), g.W, dilation_of(g, a.up, co), rt.lpr);
-#pragma unroll
-                for (int pq = 0; pq < NPQ; pq++) {
-                    float t0, t2;
-                    side.read(S + (size_t)(co * NPQ + pq) * V * rt.lpr, t0, t2);
-                    tv[co * K + pq * 3 + 0][i] = t0;
-                    tv[co * K + pq * 3 + 1][i] = own[co][pq][i];
-                    tv[co * K + pq * 3 + 2][i] = t2;
-                }
-            }
-        __syncthreads();                          // the staged rows may be overwritten from here on
-#pragma unroll
-        for (int i = 0; i < V; i++) {
-            float sum = w[0] * tv[0][i];
-#pragma unroll
-            for (int t = 1; t < KR; t++) sum += w[t] * tv[t][i];
-            gv[i] += sum;
-            if (a.masked) gv[i] = 0.f < m[i] ? gv[i] : 0.f;
-        }
-        if (act) store_vec<V>(gxp + go, gv);
-        // lanes outside the image took their side taps from the last voxel's positions: their x counts as zero
+        // lanes outside the image take their side taps from the last voxel's positions: their x counts as zero
 #pragma unroll
         for (int i = 0; i < V; i++) xv[i] = act ? xv[i] : 0.f;
+        // layer by layer, so that only one layer's nine taps per voxel are live at a time
 #pragma unroll
-        for (int t = 0; t < KR; t++)
+        for (int co = 0; co < WOUT; co++) {
+            // voxel by voxel: the twelve LDS reads of a voxel together, then its sums (the
+            // scheduling barriers keep the reads of the other voxels out of its registers)
 #pragma unroll
-            for (int i = 0; i < V; i++) ksum[t] += tv[t][i] * xv[i];
+            for (int i = 0; i < V; i++) {
+                const SideTaps<V> side(min(x0 + i, g.W - 1), g.W, dilation_of(g, a.up, co), rt.lpr);
+                float ra[NPQ][4];
+#pragma unroll
+                for (int pq = 0; pq < NPQ; pq++) {
+                    const float *srow = S + (size_t)(co * NPQ + pq) * V * rt.lpr;
+                    ra[pq][0] = srow[side.i0a];
+                    ra[pq][1] = srow[side.i0b];
+                    ra[pq][2] = srow[side.i2a];
+                    ra[pq][3] = srow[side.i2b];
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int pq = 0; pq < NPQ; pq++) {
+                    const float t[3] = {(side.m0a ? ra[pq][0] : 0.f) + (side.m0b ? ra[pq][1] : 0.f), own[co][pq][i],
+                                        (side.m2a ? ra[pq][2] : 0.f) + (side.m2b ? ra[pq][3] : 0.f)};
+#pragma unroll
+                    for (int q = 0; q < 3; q++) {
+                        gv[i] += w[co * K + pq * 3 + q] * t[q];
+                        ksum[co * K + pq * 3 + q] += t[q] * xv[i];
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        if (a.masked) {
+#pragma unroll
+            for (int i = 0; i < V; i++) gv[i] = 0.f < m[i] ? gv[i] : 0.f;
+        }
+        if (act) store_vec<V>(gxp + go, gv);
+        __syncthreads();                          // the next tile overwrites the staged rows
     }
 
     // the lanes of a wave by a fixed shuffle tree, then the waves in order
-    __syncthreads();
     const int wave = tid / kWave, wl = tid % kWave, nwaves = blockDim.x / kWave;
 #pragma unroll
     for (int t = 0; t < KR; t++) {
