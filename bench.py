@@ -115,7 +115,7 @@ def make_model(name, torch):
     return model
 
 
-def algorithmic_work(name, fused, paired=False):
+def algorithmic_work(name, fused, paired=False, triple_from=32):
     """Per-step algorithmic bytes and flops of each kernel class, fp32, per layer with C input
     and w output channels over N voxels and K = 9 or 27 taps:
     bytes: forward (C + w) N 4, backward_x (2C + 2w) N 4, backward_k+bias (C + 2w) N 4, the fused
@@ -124,12 +124,13 @@ def algorithmic_work(name, fused, paired=False):
     flops: 2 C w K N for each of forward, backward_x and backward_k (the fused pass does two).
     `fused` says which way the library ran the layers above the first (it reports a
     non-zero call count for the fused class); layer 0 needs no input gradient.
-    `paired`: the library runs the layers of a 2D block of width 1 two at a time (layers i and
-    i - 1, from the top, while i - 1 > 0): one fused pass over layer i's last input channel
-    alone, (3 + 2) N 4 bytes, and one over the c channels below both layers with the two layers
-    as its two output channels, (3c + 4) N 4 bytes: what that algorithm has to move, which is
-    about half of the per-layer figure.  The per-layer figure is returned as well, under
-    "backward_xkb_per_layer".
+    `paired`: the library runs the layers of a 2D block of width 1 in groups of n = 3 (where the
+    group's layers share at least `triple_from` channels; None: never) or 2 layers, from the top,
+    while the group's lowest layer is above layer 0: the top j layers of the group over the
+    single channel that the layer below them wrote, (3 + 2j) N 4 bytes, for j = 1 .. n - 1, and
+    one pass over the c channels below all n layers with the layers as its n output channels,
+    (3c + 2n) N 4 bytes: what that algorithm has to move, a half to a third of the per-layer
+    figure.  The per-layer figure is returned as well, under "backward_xkb_per_layer".
     Returns (bytes per class, flops per class, voxels per step)."""
     kind, ndim, c_in, c_out, depth, width, batch, spatial, adam = WORKLOADS[name]
     n = batch
@@ -143,11 +144,14 @@ def algorithmic_work(name, fused, paired=False):
     if fused and paired:
         i = depth - 1
         while i - 1 > 0:
-            in_pair.update((i, i - 1))
-            c = c_in + width * (i - 1)           # channels below both layers
-            nbytes["backward_xkb"] += (3 + 2) * n * 4 + 2 * K * 4
-            nbytes["backward_xkb"] += (3 * c + 4) * n * 4 + 2 * (2 * c * K * 4)
-            i -= 2
+            first = c_in + width * i             # channels that layer i reads
+            m = 3 if triple_from is not None and i - 2 > 0 and first - 2 >= max(triple_from, 1) else 2
+            in_pair.update(range(i - m + 1, i + 1))
+            c = first - (m - 1)                  # channels below all layers of the group
+            for j in range(1, m):
+                nbytes["backward_xkb"] += (3 + 2 * j) * n * 4 + 2 * j * K * 4
+            nbytes["backward_xkb"] += (3 * c + 2 * m) * n * 4 + 2 * (m * c * K * 4)
+            i -= m
     for i in range(depth):
         C = c_in + width * i
         wts = width * C * K * 4
@@ -269,10 +273,13 @@ def measure(name, args, lib, torch):
 
     if not args.no_kernel_timing:
         totals = kernel_times(lib, torch, lambda: [eager_step() for _ in range(args.steps)])
-        # 2D blocks of width 1 run their layers two at a time in the backward pass (block.pair)
-        paired = ndim == 2 and width == 1 and not any(kv.replace(" ", "") in ("block.pair=0", "block.fuse=0")
-                                                      for kv in args.tune)
-        bytes_per_step, flops_per_step, _ = algorithmic_work(name, totals["backward_xkb"][1] > 0, paired)
+        # 2D blocks of width 1 run their layers two or three at a time in the backward pass
+        # (block.pair; block.triple: from how many shared channels three, 0 never, 32 by default)
+        tuned = dict(kv.replace(" ", "").split("=") for kv in args.tune)
+        paired = ndim == 2 and width == 1 and tuned.get("block.pair") != "0" and tuned.get("block.fuse") != "0"
+        triple = int(tuned.get("block.triple", -1))
+        triple_from = None if triple == 0 else (32 if triple < 0 else triple)
+        bytes_per_step, flops_per_step, _ = algorithmic_work(name, totals["backward_xkb"][1] > 0, paired, triple_from)
         kernels = {}
         for cls, (ms, launches) in totals.items():
             if launches == 0:
@@ -290,7 +297,7 @@ def measure(name, args, lib, torch):
             if cls == "backward_xkb" and paired:
                 # the same time priced with the bytes of one fused pass per layer, for comparison
                 per_layer = bytes_per_step["backward_xkb_per_layer"]
-                kernels[cls]["layers_in_pairs"] = True
+                kernels[cls]["layers_in_groups"] = True
                 kernels[cls]["per_layer_GB_per_step"] = round(per_layer / 1e9, 3)
                 kernels[cls]["per_layer_GBps"] = round(per_layer / per_step_s / 1e9, 1)
         dominant = max(kernels, key=lambda c: kernels[c]["ms_per_step"])

@@ -140,10 +140,14 @@ __global__ __launch_bounds__(kThreads, 4) void bwd_one_channel(const Args a, con
 
 // Voxels per lane, or 0: rows of whole waves that one team of at most 256 lanes covers,
 // naturally aligned V-wide accesses in all three tensors.
+// Two layers come with a pass of three layers over the other channels, which takes rows of whole
+// groups of four voxels only: such rows never need one voxel per lane.
+inline int min_vec(const Geom &g) { return g.Wd == 2 ? 2 : 1; }
+
 int choose_vec(const Geom &g, const View<const float> &gy, const View<const float> &x, const View<float> &gx,
                RowTeams *rt)
 {
-    for (int v = 4; v >= 1; v /= 2) {
+    for (int v = 4; v >= min_vec(g); v /= 2) {
         if (!rows_aligned(gy, g.W, v) || !rows_aligned(x, g.W, v) || !rows_aligned(gx, g.W, v)) continue;
         if (!make_row_teams(g, v, rt)) continue;
         if (rt->lpr % kWave != 0 || rt->lpr * rt->rpw > kThreads) continue;
@@ -179,7 +183,7 @@ static void launch_one_channel(int v, dim3 grid, dim3 block, size_t lds, hipStre
         hipLaunchKernelGGL((bwd1::bwd_one_channel<4, WOUT>), grid, block, lds, s, a, gy, x, gx, act, k, k1, part);
     else if (v == 2)
         hipLaunchKernelGGL((bwd1::bwd_one_channel<2, WOUT>), grid, block, lds, s, a, gy, x, gx, act, k, k1, part);
-    else
+    else if constexpr (WOUT == 1)     // (two layers: see min_vec)
         hipLaunchKernelGGL((bwd1::bwd_one_channel<1, WOUT>), grid, block, lds, s, a, gy, x, gx, act, k, k1, part);
 }
 

@@ -215,6 +215,7 @@ PAIR_BLOCKS = [
     ((20, 255), 1, 5, 1, [2, 7, 1, 4, 3]),          # odd rows: one voxel per lane in the one-channel step
     ((40, 64), 1, 20, 1, None),
     ((10, 384), 1, 7, 1, [3, 1, 4, 1, 5, 9, 2]),    # two voxels per lane in the one-channel steps
+    ((9, 192), 2, 6, 1, [1, 3, 2, 4, 1, 2]),        # one voxel per lane in the one-channel steps
     ((8, 1280), 40, 6, 1, [2, 7, 1, 8, 2, 8]),      # three layers over more than 32 channels (the default's threshold)
     ((6, 512), 70, 3, 2, [6, 1, 3]),                # three layers, channels in two chunks of the grid
 ]
@@ -230,6 +231,21 @@ def test_block_backward_two_or_three_layers_at_a_time(case, grouping):
     size, c_in, depth, batch, dilations = case
     with tuning(GROUPINGS[grouping]):
         check_block(2, size, c_in, 1, depth, batch, dilations=dilations, seed=11)
+
+
+def _random_one_channel_blocks(n):
+    from test_random_shapes_gpu import _block_cases
+    return [c for c in _block_cases(4242, 80) if c[0] == 2 and c[3] == 1 and c[4] >= 5][:n]
+
+
+@pytest.mark.parametrize("case", _random_one_channel_blocks(12), ids=lambda c: "%s-c%d-depth%d-B%d" % (
+    "x".join(map(str, c[1])), c[2], c[4], c[5]))
+def test_random_blocks_three_layers_at_a_time(case):
+    # seeded random 2D blocks of one-channel layers (ragged and odd rows among them: where the
+    # three-layer kernels do not apply the walk falls back to two layers or one)
+    import test_random_shapes_gpu
+    with tuning({"block.triple": 1}):
+        test_random_shapes_gpu.test_random_blocks(case)
 
 
 def test_paired_and_single_backward_agree_when_the_input_needs_no_gradient():
