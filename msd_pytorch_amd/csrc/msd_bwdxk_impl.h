@@ -126,7 +126,9 @@ void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *_
     // 16-voxel MFMA groups per pipeline stage, by measurement: 32 voxels in 2D with four voxels
     // per lane, 16 voxels in 3D up to 64 channels per chunk (these instances then fit the
     // registers of three workgroups per CU without spills), 64 voxels with two voxels per lane
-    constexpr int NSS = V == 1 ? (NCB <= 4 ? 1 : 2) : (V == 4 ? 2 : 4);
+    // (32 with three output channels: the pipeline buffers of 64 would push the accumulators of
+    // 128 channels out of the registers)
+    constexpr int NSS = V == 1 ? (NCB <= 4 ? 1 : 2) : (V == 4 || WOUT == 3 ? 2 : 4);
     constexpr int H = 4 * V / NSS;                // stages per block of 16 channels (even)
     constexpr int NCS = kChanBlock / H;           // grad_input channels per stage
     constexpr int NSETS = pipeline_sets<NDIM, V, NCB, WOUT, LONG>();   // register sets of the load pipeline
@@ -785,14 +787,8 @@ hipError_t pick_ncb(const Geom &g, const View<const float> &gy, const View<const
     const int need = (g.C + kChanBlock - 1) / kChanBlock;
     if (need <= 1) return launch<NDIM, V, 1, WOUT, LONG, BIG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, group);
     if (need <= 2) return launch<NDIM, V, 2, WOUT, LONG, BIG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, group);
-    // (three output channels: more than 64 channels per chunk do not fit the registers; the
-    // channels then go in chunks of 64 over the grid's third dimension)
-    if constexpr (WOUT >= 3) {
-        return launch<NDIM, V, 4, WOUT, LONG, BIG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, group);
-    } else {
-        if (need <= 4) return launch<NDIM, V, 4, WOUT, LONG, BIG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, group);
-        return launch<NDIM, V, 8, WOUT, LONG, BIG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, group);
-    }
+    if (need <= 4) return launch<NDIM, V, 4, WOUT, LONG, BIG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, group);
+    return launch<NDIM, V, 8, WOUT, LONG, BIG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, group);
 }
 
 // Widest vector for two output channels (2D only): twice the gathered values per voxel must
