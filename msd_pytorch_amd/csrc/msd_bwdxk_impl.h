@@ -77,9 +77,9 @@ struct Args {
 };
 
 // The waves' tiles share the LDS of the staged rows (two outputs at four voxels per lane: the
-// tiles alone are 79 KB).
+// tiles alone are 79 KB; three outputs, or 3D at two voxels per lane: 59 KB).
 template <int NDIM, int V, int WOUT>
-constexpr bool tiles_over_staging() { return NDIM == 2 && ((V == 4 && WOUT == 2) || WOUT == 3); }
+constexpr bool tiles_over_staging() { return (NDIM == 2 && ((V == 4 && WOUT == 2) || WOUT == 3)) || (NDIM == 3 && V == 2); }
 
 // Workgroups (of four waves) that are resident per CU.  The 3D kernel with one voxel per lane
 // (pipeline stages of 16 voxels, arguments read again per tile, row arithmetic on the scalar
@@ -686,7 +686,7 @@ bool fits(const Geom &g, int V, const View<const float> &gy, const View<const fl
     const size_t kr = (size_t)g.Wd * Taps<NDIM>::K + 1;
     const size_t staged = (size_t)rt.rpw * g.Wd * RowTaps<NDIM>::NPQ * (V * rt.lpr + sg.halo) * 4;
     const size_t tiles = (size_t)kWaves * kr * (kWave * V + 4) * 4;
-    const bool over = NDIM == 2 && ((V == 4 && g.Wd == 2) || g.Wd == 3);   // tiles_over_staging()
+    const bool over = (NDIM == 2 && ((V == 4 && g.Wd == 2) || g.Wd == 3)) || (NDIM == 3 && V == 2);   // tiles_over_staging()
     if ((over ? std::max(staged, tiles) : staged + tiles) > (over ? kMaxLdsBytesAsked : kMaxLdsBytes)) return false;
     return rows_aligned(gy, g.W, V) && rows_aligned(gx, g.W, V);
 }
@@ -695,9 +695,10 @@ template <int NDIM>
 int choose_vec(const Geom &g, int vmax, const View<const float> &gy, const View<const float> &x,
                const View<float> &gx, bool lng)
 {
-    // 3D: one voxel per lane only (27 gathered taps per voxel; the staged rows and the waves'
-    // tiles of two voxels per lane do not fit the LDS budget at any row length)
-    for (int v = NDIM == 3 ? 1 : 4; v >= 1; v /= 2) {
+    // 3D: one voxel per lane where that covers the row (27 gathered taps per voxel: twice the
+    // resident waves, 10 % faster at 128^3); two, with the waves' tiles over the staged rows, for
+    // rows of 257 to 512 voxels, which otherwise go in segments (15-20 % slower)
+    for (int v = NDIM == 3 ? (lng ? 1 : 2) : 4; v >= 1; v /= 2) {
         if (v > vmax) continue;
         if (fits<NDIM>(g, v, gy, x, gx, lng)) return v;
     }
@@ -898,6 +899,9 @@ hipError_t xkb_nd(const Geom &g, const View<const float> &gy, const View<const f
     if (g.Wd != 1) return hipErrorInvalidConfiguration;
     if constexpr (NDIM == 2) {
         if (v == 2) return pick_ncb<2, 2, 1, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, nullptr);
+    }
+    if constexpr (NDIM == 3 && !LONG) {
+        if (v == 2) return pick_ncb<3, 2, 1, false>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, nullptr);
     }
     if (v == 1) return pick_ncb<NDIM, 1, 1, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, nullptr);
     return hipErrorInvalidConfiguration;

@@ -164,6 +164,13 @@ INSTANCES = [
     ({}, (1, 40, 3, (5, 2048), 2)),
     ({}, (1, 130, 3, (6, 1024), 5)),
     ({}, (1, 20, 3, (7, 1026), 3)),                  # not covered by the fused kernel: two passes
+    # 3D rows of 257 to 512 voxels: the fused backward at two voxels per lane (tiles over the
+    # staged rows), by channel blocks
+    ({}, (1, 9, 1, (3, 4, 512), 3)),
+    ({}, (2, 20, 1, (4, 3, 384), 2)),
+    ({}, (1, 40, 1, (3, 5, 512), 1)),
+    ({}, (1, 70, 1, (2, 4, 512), 2)),
+    ({"bwdk.vec3d": 2}, (1, 20, 1, (5, 6, 128), 2)),
 ]
 
 
