@@ -37,6 +37,9 @@
 #ifndef MSD_XPAIR
 #define MSD_XPAIR 1
 #endif
+#ifndef MSD_INNER_PATH
+#define MSD_INNER_PATH 1
+#endif
 #ifndef MSD_PIPELINE_SETS_EXPR
 #define MSD_PIPELINE_SETS_EXPR 2
 #endif
@@ -142,6 +145,9 @@ void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *_
     static_assert(!XPAIR || (H == 4 && NSETS == 2), "a block is two pairs of stages");
     static_assert(H % NSETS == 0 && NSETS >= 2, "the stages of a block rotate through the register sets");
     constexpr int ASTRIDE = ATile<NDIM, V, WOUT>::kStride;
+    // 2D: waves away from the row ends take their x-taps without the mirror arithmetic (3D rows
+    // are short: every wave touches an end)
+    constexpr bool INNER_PATH = NDIM == 2 && MSD_INNER_PATH;
     const Args &a = a_;
     const Geom &g = a.g;
     const RowTeams &rt = a.rt;
@@ -332,6 +338,8 @@ void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *_
             } else {
                 stage_source_rows<NDIM, false, WOUT, V>(g, rt, none, gyv, b, zc, yc, lane, act, S, own, a.up);
             }
+            // the voxels of this wave: [xw, xw + 64 V) (uniform)
+            const int xw = __builtin_amdgcn_readfirstlane(x0);
             // per voxel: all LDS reads first, so that their latencies overlap, then the sums
 #pragma unroll
             for (int i = 0; i < V; i++)
@@ -339,6 +347,34 @@ void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *_
                 for (int co = 0; co < WOUT; co++) {
                     // (the upper output channels may have dilations of their own, and with them their own x-taps)
                     const int dil = dilation_of(g, a.up, co);
+                    if (INNER_PATH && xw >= dil && xw + kWave * V + dil <= g.W) {
+                        // no lane of the wave is within `dil` of a row end: both x-taps of every
+                        // voxel lie inside the row (no mirrored source, nothing to mask): two LDS
+                        // reads per staged row instead of four
+                        auto at = [&](int p) {    // LDS position of the row's voxel p
+                            const int j = p - xs, segw = V * rt.lpr;
+                            if (!segmented) return staged_index<V>(p, rt.lpr);
+                            return j < 0 ? segw + (j + dil) : (j >= segw ? segw + dil + (j - segw) : staged_index<V>(j, rt.lpr));
+                        };
+                        const int ihi = at(x0 + i + dil), ilo = at(x0 + i - dil);
+                        float rb[NPQ][2];
+#pragma unroll
+                        for (int pq = 0; pq < NPQ; pq++) {
+                            const float *srow = S + (size_t)(co * NPQ + pq) * rs;
+                            rb[pq][0] = srow[ihi];
+                            rb[pq][1] = srow[ilo];
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                        for (int pq = 0; pq < NPQ; pq++) {
+                            const int r = co * NPQ + pq;
+                            tv[r * 3 + 0][i] = rb[pq][0];
+                            tv[r * 3 + 1][i] = own[co][pq][i];
+                            tv[r * 3 + 2][i] = rb[pq][1];
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+                        continue;
+                    }
                     const SideTaps<V> side = segmented ? SideTaps<V>(x0 + i, g.W, dil, rt.lpr, xs, V * rt.lpr)
                                                        : SideTaps<V>(min(x0 + i, g.W - 1), g.W, dil, rt.lpr);
                     float ra[NPQ][4];
