@@ -32,6 +32,7 @@
 #pragma once
 #include "msd_bwdk_impl.h"
 
+#include <atomic>
 #include <type_traits>
 
 #ifndef MSD_XPAIR
@@ -790,9 +791,19 @@ hipError_t launch(const Geom &g, const View<const float> &gy, const View<const f
     constexpr bool kAsks = tiles_over_staging<NDIM, V, WOUT>();
     if (lds > (kAsks ? kMaxLdsBytesAsked : kMaxLdsBytes)) return hipErrorInvalidConfiguration;   // excluded by fits()
     if (kAsks && lds > kMaxLdsBytes) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&bwd_rows_fused<NDIM, V, NCB, WOUT, LONG, BIG>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLdsBytesAsked);
+        // more than 64 KB has to be asked for, once per kernel and device (the attribute stays):
+        // later launches, also ones recorded into a graph, go without the call
+        static std::atomic<uint64_t> asked{0};
+        int dev = 0;
+        hipError_t e = hipGetDevice(&dev);
         if (e != hipSuccess) return e;
+        const uint64_t bit = dev >= 0 && dev < 64 ? (uint64_t)1 << dev : 0;
+        if (!(asked.load(std::memory_order_acquire) & bit)) {
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(&bwd_rows_fused<NDIM, V, NCB, WOUT, LONG, BIG>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLdsBytesAsked);
+            if (e != hipSuccess) return e;
+            asked.fetch_or(bit, std::memory_order_release);
+        }
     }
     // the weights of the upper output channels follow those of the first, or are other layers'
     const float *k1 = group ? group->k_up[0] : k + (int64_t)g.C * K;

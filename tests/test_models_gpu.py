@@ -417,13 +417,15 @@ def test_gradients_and_learn_report_the_forward_loss():
     assert model.forward(x, y) != loss                         # the update moved the parameters
 
 
-@pytest.mark.parametrize("kind,ndim", [("regression", 2), ("segmentation", 2), ("regression", 3)])
-def test_step_replayed_from_a_hip_graph_equals_the_eager_step(kind, ndim):
+@pytest.mark.parametrize("kind,ndim,size", [("regression", 2, (48, 96)), ("segmentation", 2, (48, 96)),
+                                            ("regression", 3, (6, 10, 64)), ("regression", 2, (6, 1024))],
+                         ids=["regression-2d", "segmentation-2d", "regression-3d", "regression-2d-rows-of-1024"])
+def test_step_replayed_from_a_hip_graph_equals_the_eager_step(kind, ndim, size):
     # every replay is checked against the eager step on the same data, with eager work and
-    # synchronisations between the replays
+    # synchronisations between the replays (rows of 1024 voxels: the backward kernels that ask
+    # for more than 64 KB of LDS)
     from msd_pytorch_amd import GraphedStep, MSDRegressionModel, MSDSegmentationModel
     torch.manual_seed(11)
-    size = (48, 96) if ndim == 2 else (6, 10, 64)
     dil = [1, 2, 3, 4, 5]
     if kind == "regression":
         model = MSDRegressionModel(2, 1, depth=9, width=1, dilations=dil, ndim=ndim)
