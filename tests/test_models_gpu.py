@@ -71,7 +71,7 @@ FUSED_BLOCK_CASES = [
     (2, (21, 128), 2, 11, 1, None, 2),     # width 2: two output channels per layer in the fused pass
     (2, (300, 132), 2, 4, 2, None, 2),     # width 2, several tiles per workgroup
     (2, (23, 2048), 1, 5, 2, [1, 2, 9, 23, 4]),      # rows of 2 segments of 1024 voxels
-    (2, (19, 1536), 2, 3, 1, [3, 1, 10], 2),       # width 2, rows of 3 segments of 512 voxels
+    (2, (19, 1536), 2, 3, 1, [3, 1, 10], 2),       # width 2, rows of 2 segments (1024 and 512 voxels)
     (2, (11, 750), 1, 4, 1, None),         # rows that are not whole groups of four voxels
     (2, (6, 1001), 2, 3, 2, [1, 5, 3], 2),   # odd rows, width 2
     (3, (5, 6, 130), 1, 3, 1, None),       # the same in 3D

@@ -179,8 +179,8 @@ SHAPES_XKB = [
     (2, 18, 1, (7, 2048), 5),         # 2 channel blocks, folds in y
     (1, 4, 1, (130, 1536), 128),      # 3 segments of 512, the largest dilation the halo takes
     (1, 2, 1, (140, 2048), 129),      # dilation past that: the separate kernels
-    (1, 5, 2, (8, 1024), 7),          # two output channels: 2 segments of 512
-    (1, 3, 2, (4, 2048), 3),          # two output channels: 4 segments
+    (1, 5, 2, (8, 1024), 7),          # two output channels: four voxels per lane, one tile per row
+    (1, 3, 2, (4, 2048), 3),          # two output channels: 2 segments of 1024
     # rows that are not whole groups of four voxels (unaligned rows of the input stack)
     (1, 3, 1, (6, 750), 2),           # 2 voxels per lane, a short second segment
     (2, 18, 1, (5, 1001), 3),         # odd: one voxel per lane, 4 segments
@@ -189,8 +189,8 @@ SHAPES_XKB = [
     (1, 4, 1, (9, 250), 3),           # whole rows per team, the last group of four is half empty
     (1, 7, 1, (5, 6, 130), 2),        # 3D
     (1, 3, 1, (4, 5, 127), 1),        # 3D, odd
-    (1, 3, 1, (4, 5, 512), 3),        # 3D rows of two segments
-    (2, 18, 1, (3, 4, 300), 2),       # 3D, a short second segment, folds in z and y
+    (1, 3, 1, (4, 5, 512), 3),        # 3D rows of 512 voxels: two voxels per lane
+    (2, 18, 1, (3, 4, 300), 2),       # 3D, two voxels per lane, lanes past the row's end, folds in z and y
 ]
 
 
