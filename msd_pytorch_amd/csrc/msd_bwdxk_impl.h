@@ -66,6 +66,17 @@ struct Plane {
     int sb, sc, sz, sy;
 };
 
+// One step of a workgroup from tile to tile (group_step tiles ahead), taken apart on the host so
+// that the kernel advances its position with additions and compares only: in segments of a row,
+// row groups of an image and batch items; the row groups again as rows, split into y and z; and
+// the rows of a wrap to the next batch item (ngroups * rpw) and of a carried segment (rpw).
+struct TileStep {
+    int seg, gi, b;
+    int y, z;
+    int wrap_y, wrap_z;
+    int carry_y, carry_z;
+};
+
 struct Args {
     Geom g;
     RowTeams rt;
@@ -78,6 +89,7 @@ struct Args {
     int want_bias;
     RowSegments sg;      // LONG instances
     UpperDilations up;   // layers of a dense block in one pass: the dilations of output channels 1 and 2
+    TileStep step;
 };
 
 // The waves' tiles share the LDS of the staged rows (two outputs at four voxels per lane: the
@@ -202,8 +214,8 @@ void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *_
 #pragma unroll
     for (int tg = 0; tg < TG; tg++) arow[tg] = min(tg * 16 + mj, KR) * ASTRIDE + 4 * mk;
 
-    // Position of the lane's row, advanced from tile to tile without divisions: the row groups
-    // of a workgroup are consecutive.
+    // Position of the lane's row: divisions here, once; from tile to tile it advances by
+    // additions and compares (Args::step).
     int grp = a.group_step == 1 ? lb * a.tiles_per_wg : lb;
     int seg = 0, rg = grp;                                    // uniform: segment of the row, row group
     if constexpr (SEG) {
@@ -212,7 +224,9 @@ void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *_
     }
     int gi = rg % a.ngroups, b = rg / a.ngroups;              // uniform: group within the image, batch index
     int row = gi * rt.rpw + team;
-    int y = row % g.H, z = row / g.H;
+    // 3D: (y0, z0) is the first row of the group; 2D: a row is its own y
+    int y0 = NDIM == 3 ? (gi * rt.rpw) % g.H : 0, z0 = NDIM == 3 ? (gi * rt.rpw) / g.H : 0;
+    int y = NDIM == 3 ? row % g.H : row, z = NDIM == 3 ? row / g.H : 0;
 
     // The kernel's arguments are the first thing in the argument block.  The 3D instances read
     // them again from there for every tile (scalar loads) instead of keeping them over the
@@ -604,35 +618,48 @@ void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *_
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         if constexpr (ALIAS) __syncthreads();     // the next tile's staged rows overwrite every wave's tile
-        // next row group
-        if (a.group_step != 1 || SEG) {           // uniform
-            grp += a.group_step;
-            rg = grp;
-            if constexpr (SEG) {
-                seg = grp % a.sg.segs;
-                rg = grp / a.sg.segs;
+        // next tile (all of this is uniform)
+        grp += a.group_step;
+        int carry = 0;
+        if constexpr (SEG) {
+            seg += a.step.seg;
+            if (seg >= a.sg.segs) {
+                seg -= a.sg.segs;
+                carry = 1;
             }
-            gi = rg % a.ngroups;
-            b = rg / a.ngroups;
-            row = gi * rt.rpw + team;
-            y = row % g.H;
-            z = row / g.H;
-            continue;
         }
-        grp++;
-        if (++gi == a.ngroups) {                  // uniform: first group of the next batch item
-            gi = 0;
+        gi += a.step.gi + carry;
+        b += a.step.b;
+        if constexpr (NDIM == 3) {
+            y0 += a.step.y + (carry ? a.step.carry_y : 0);
+            z0 += a.step.z + (carry ? a.step.carry_z : 0);
+        }
+        if (gi >= a.ngroups) {                    // into the next batch item
+            gi -= a.ngroups;
             b++;
-            row = team;
-            y = team % g.H;
-            z = team / g.H;
-        } else {
-            row += rt.rpw;
-            y += rt.rpw;
+            if constexpr (NDIM == 3) {
+                y0 -= a.step.wrap_y;
+                z0 -= a.step.wrap_z;
+            }
+        }
+        row = gi * rt.rpw + team;
+        if constexpr (NDIM == 3) {
+            while (y0 >= g.H) {
+                y0 -= g.H;
+                z0++;
+            }
+            while (y0 < 0) {
+                y0 += g.H;
+                z0--;
+            }
+            y = y0 + team;
+            z = z0;
             while (y >= g.H) {
                 y -= g.H;
                 z++;
             }
+        } else {
+            y = row;
         }
     }
 
@@ -780,6 +807,18 @@ hipError_t launch(const Geom &g, const View<const float> &gy, const View<const f
         a.tiles_per_wg = (int)((total + rows - 1) / rows);
     }
     a.total_groups = (int)total;
+    {
+        const int s_rg = a.group_step / a.sg.segs, rows_step = (a.group_step / a.sg.segs % a.ngroups) * a.rt.rpw;
+        a.step.seg = a.group_step % a.sg.segs;
+        a.step.gi = s_rg % a.ngroups;
+        a.step.b = s_rg / a.ngroups;
+        a.step.y = rows_step % g.H;
+        a.step.z = rows_step / g.H;
+        a.step.wrap_y = (a.ngroups * a.rt.rpw) % g.H;
+        a.step.wrap_z = (a.ngroups * a.rt.rpw) / g.H;
+        a.step.carry_y = a.rt.rpw % g.H;
+        a.step.carry_z = a.rt.rpw / g.H;
+    }
     a.gy = Plane{(int)gy.sb, (int)gy.sc, (int)gy.sz, (int)gy.sy};
     a.x = Plane{(int)x.sb, (int)x.sc, (int)x.sz, (int)x.sy};
     a.gx = Plane{(int)gx.sb, (int)gx.sc, (int)gx.sz, (int)gx.sy};
