@@ -875,6 +875,10 @@ hipError_t pick_ncb(const Geom &g, const View<const float> &gy, const View<const
     if (need <= 1) return launch<NDIM, V, 1, WOUT, LONG, BIG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, group);
     if (need <= 2) return launch<NDIM, V, 2, WOUT, LONG, BIG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, group);
     if (need <= 4) return launch<NDIM, V, 4, WOUT, LONG, BIG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, group);
+    if constexpr (WOUT == 3) {
+        // three output channels: the accumulators of 128 channels spill a few registers, those of 96 do not
+        if (need <= 6) return launch<NDIM, V, 6, WOUT, LONG, BIG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, group);
+    }
     return launch<NDIM, V, 8, WOUT, LONG, BIG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, group);
 }
 

@@ -171,6 +171,7 @@ INSTANCES = [
     ({}, (1, 40, 1, (3, 5, 512), 1)),
     ({}, (1, 70, 1, (2, 4, 512), 2)),
     ({"bwdk.vec3d": 2}, (1, 20, 1, (5, 6, 128), 2)),
+    ({}, (1, 40, 1, (4, 5, 130), 2)),                # 3D rows that are not whole groups of four voxels, 33-64 channels
 ]
 
 
