@@ -1,7 +1,10 @@
 // backward_x and backward_k (+ bias) of one layer in a single pass over the input
-// channels, fp32, unit x-stride, one output channel, output gradient already masked:
+// channels, fp32, unit x-stride, output gradient already masked:
 //     grad_input[ci][u] += sum_t k[ci][t] * A[t](u)
 //     grad_kernel[ci][t] += sum_u x[ci][u] * A[t](u),     grad_bias += sum_u A[centre](u)
+// for one output channel, or summed over / repeated for two or three (2D): the output
+// channels of one layer, or two or three one-channel layers of a dense block with their own
+// dilations, weights and gradients, which share the input channels of the lowest of them.
 // Both need the same adjoint-form gather A[t](u) of the output gradient (msd_adjoint.h,
 // msd_rows.h); done once per tile of rows, it then serves a stream over the input
 // channels that reads x[ci], reads and writes grad_input[ci], and touches nothing else.
