@@ -272,8 +272,9 @@ __global__ __launch_bounds__(kFinalThreads) void final_forward_loss_kernel(
         sb = wave_sum(sb);
         if (lane == 0 && o < c_out) part[((int64_t)c_out * C + o) * rows + row] = sb;
     }
+    // (from the last channel to the first: what the first walk read last is still in the caches)
 #pragma unroll 2
-    for (int c = 0; c < C; c++) {
+    for (int c = C - 1; c >= 0; c--) {
         T v[V];
         load_elems<T, V>(xp + (int64_t)c * xsc, v);
 #pragma unroll
