@@ -20,8 +20,8 @@ import numpy as np
 import torch
 from torch.utils.data import DataLoader
 
-import msd_pytorch_amd as mp
-from msd_pytorch_amd.image_dataset import write_tiff
+import msd_pytorch as mp
+from msd_pytorch.image_dataset import write_tiff
 
 
 def write_synthetic_set(folder, count, size, num_labels, seed):

@@ -121,19 +121,28 @@ class GraphedStep:
             raise ValueError("GraphedStep: call set_input and set_target first")
         self.model = model
         model.loss = model.output = None          # no autograd graph of an earlier step kept alive
+        # the graph's static buffers are its own: set_input / set_target keep a tensor that is
+        # already on the GPU as it is, and every replay overwrites these
+        model.input, model.target = model.input.clone(), model.target.clone()
+        # warm-up and capture run on ONE side stream: the gradient accumulators of the
+        # parameters are made in the first backward pass and stay with the stream they were made on
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
             for _ in range(warmup):
                 model.step_async(update=update)
+            model.loss = model.output = None
+            model.optimizer.zero_grad(set_to_none=True)
         torch.cuda.current_stream().wait_stream(side)
-        model.optimizer.zero_grad(set_to_none=True)
         self.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(self.graph):
+        with torch.cuda.graph(self.graph, stream=side):
             model.step_async(update=update)
         self._input, self._target = model.input, model.target
         self.shapes = (model.input.shape, model.target.shape)
-        self._loss, self._output = model.loss, model.output
+        # the values only: the recorded autograd graph would keep the parameters' gradient
+        # accumulators (and their stream) alive for every eager step that follows
+        self._loss, self._output = model.loss.detach(), model.output.detach()
+        model.loss, model.output = self._loss, self._output
         # the gradient tensors the graph writes (an eager step in between replaces .grad)
         self._grads = [(p, p.grad) for group in model.optimizer.param_groups for p in group["params"]
                        if p.grad is not None]
@@ -202,7 +211,7 @@ class MSDModel:
             self.set_target(target)
         self.output = None
         self.loss = None
-        fused = self._fused_forward_loss() if self.fuse_loss else None
+        fused = self._fused_forward_loss() if self.fuse_loss and not self._net_hooked() else None
         if fused is not None:
             self.loss, self.output = fused
             return
@@ -211,7 +220,18 @@ class MSDModel:
 
     # Loss computed in the pass of the final layer (MSDModule.forward_loss) where the model has
     # the standard structure; set to False to run network and criterion as separate modules.
+    # With the fused node ``model.output`` is detached from the autograd graph: a further loss
+    # built on it gets no gradient.  Hooks on any module of ``net`` switch the fusion off for
+    # that call, since the hooks' modules are then not called one by one.
     fuse_loss = True
+
+    def _net_hooked(self):
+        """True when any module of ``net`` (the Sequential containers, the scaling layers, the
+        MSD module and its parts, LogSoftmax) carries a forward, pre-forward or backward hook."""
+        for m in self.net.modules():
+            if m._forward_hooks or m._forward_pre_hooks or m._backward_hooks or m._backward_pre_hooks:
+                return True
+        return False
 
     def _loss_kind(self):
         """"mse", "l1" or "nll" when the criterion is torch's with default settings, else None."""
@@ -266,20 +286,32 @@ class MSDModel:
         (depth 10 at 256 x 256: 0.25 against 0.7 ms per step).  The optimiser is then switched
         to its capturable form, keeping its state."""
         # the loss of each batch is not looked at here (the reference drops it too):
-        # the host keeps launching ahead of the GPU
-        step = None
+        # the host keeps launching ahead of the GPU; targets that are on the GPU already are
+        # validated there and the verdict is read once per epoch (_set_target_deferred)
+        steps = {}        # one recorded step per batch shape (a loader's last batch may be smaller)
         for _ in range(num_epochs):
             for input, target in dataloader:
-                if not graph:
-                    self.step_async(input, target)
-                    continue
                 self.set_input(input)
-                self.set_target(target)
-                if step is None or step.shapes != (self.input.shape, self.target.shape):
+                self._set_target_deferred(target)
+                if not graph:
+                    self.step_async()
+                    continue
+                shapes = (self.input.shape, self.target.shape)
+                step = steps.get(shapes)
+                if step is None:
                     self._make_optimizer_capturable()
-                    step = GraphedStep(self, update=True, warmup=1)    # the warm-up run is this batch's step
+                    steps[shapes] = GraphedStep(self, update=True, warmup=1)   # the warm-up run is this batch's step
                 else:
                     step(self.input, self.target)
+            self._raise_deferred_target_error()
+
+    def _set_target_deferred(self, target):
+        """set_target for a training loop that must not wait for the GPU per batch.  Models whose
+        set_target inspects values (segmentation labels) override this for GPU tensors."""
+        self.set_target(target)
+
+    def _raise_deferred_target_error(self):
+        pass
 
     def _make_optimizer_capturable(self):
         if self.optimizer.defaults.get("capturable", False):

@@ -102,7 +102,9 @@ class MSDNetLossFunction(torch.autograd.Function):
     also computes the loss, its gradient with respect to the layer's output and the layer's own
     parameter gradients, so the backward pass starts from a tensor of c_out channels and never
     reads the stack for the final layer again.  ``output`` is returned for the caller's use and
-    is not differentiable; the scaling layer's parameters get no gradient (they are frozen in
+    is NOT differentiable (a loss of the caller's own built on it gets no gradient: run the
+    modules one by one for that, ``MSDModel.fuse_loss = False``); the scaling layer's parameters
+    get no gradient (they are frozen in
     the models, msd_model.py:8-45)."""
 
     @staticmethod
@@ -232,7 +234,8 @@ class MSDModule(torch.nn.Module):
         that is being trained."""
         linear = self.final_layer.linear
         if not (cc.final_layer_supported(input) and input.dim() in (4, 5) and input.dtype == linear.weight.dtype
-                and linear.bias is not None and not self._hooked() and self.c_out <= 8 and target.is_cuda):
+                and linear.bias is not None and not self._hooked() and self.c_out <= 8
+                and target.device == input.device):
             return None
         sw = sb = None
         if scale is not None:

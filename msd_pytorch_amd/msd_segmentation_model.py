@@ -1,4 +1,5 @@
 """MSD network for segmentation (reference msd_segmentation_model.py:10-119)."""
+import torch
 import torch.nn as nn
 
 from .msd_model import MSDModel, _moments, scaling_module_set_bias, scaling_module_set_scale
@@ -28,6 +29,8 @@ class MSDSegmentationModel(MSDModel):
         scaling_module_set_bias(self.scale_in, -mean / std)
 
     def set_target(self, target):
+        """Labels in [0, num_labels), checked here as msd_segmentation_model.py:105-119 does (for
+        a tensor on the GPU that read-back waits for the device; ``train`` defers it)."""
         target = target.long()
         lo, hi = target.min(), target.max()
         if lo < 0 or self.num_labels <= hi:
@@ -35,6 +38,26 @@ class MSDSegmentationModel(MSDModel):
                 f"Target invalid: expected values in range {[0, self.num_labels - 1]}, but got {[lo, hi]}")
         # NLLLoss takes (B, *spatial) class indices: drop the channel axis
         self.target = target.squeeze(1).cuda()
+
+    def _set_target_deferred(self, target):
+        if not target.is_cuda:
+            return self.set_target(target)      # a host tensor is checked on the host: no device wait
+        target = target.long()
+        # lowest and highest label seen since the last verdict, kept on the device; the step
+        # itself runs on labels clamped into range, so no loss kernel ever sees an invalid one
+        lo, hi = target.min(), target.max()
+        seen = getattr(self, "_label_range", None)
+        self._label_range = (lo, hi) if seen is None else (torch.minimum(seen[0], lo), torch.maximum(seen[1], hi))
+        self.target = target.squeeze(1).clamp(0, self.num_labels - 1)
+
+    def _raise_deferred_target_error(self):
+        seen, self._label_range = getattr(self, "_label_range", None), None
+        if seen is None:
+            return
+        lo, hi = int(seen[0]), int(seen[1])
+        if lo < 0 or self.num_labels <= hi:
+            raise ValueError(
+                f"Target invalid: expected values in range {[0, self.num_labels - 1]}, but got {[lo, hi]}")
 
     def _fused_forward_loss(self):
         if self._loss_kind() != "nll" or not isinstance(self.net, nn.Sequential) or len(self.net) != 2:

@@ -58,6 +58,15 @@ def make_problem(shape, dtype, device="cpu", seed=0):
                 k=k, bias=bias, d=d, C=C, Wd=Wd)
 
 
+def problem_on(problem, device):
+    """The same problem (same values) on another device, with the same aliasing of the
+    channel slices."""
+    C = problem["C"]
+    stack, gstack = problem["stack"].to(device), problem["gstack"].to(device)
+    return dict(stack=stack, gstack=gstack, x=stack[:, :C], y=stack[:, C:], gx=gstack[:, :C], gy=gstack[:, C:],
+                k=problem["k"].to(device), bias=problem["bias"].to(device), d=problem["d"], C=C, Wd=problem["Wd"])
+
+
 def rel_err(got, want):
     """max |got - want| / max |want|: the parity measure of every tolerance in these tests."""
     got, want = got.detach().double().cpu(), want.detach().double().cpu()

@@ -5,7 +5,7 @@ Tolerances (max |diff| / max |ref|, fp32): forward 1e-5, gradients 1e-4."""
 import torch
 
 import oracle
-from cases import make_problem, rel_err
+from cases import make_problem, problem_on, rel_err
 
 
 def bias_close(got, want, terms, tol=1e-4):
@@ -16,12 +16,14 @@ def bias_close(got, want, terms, tol=1e-4):
     return diff <= tol * max(want.abs().max().item(), floor)
 
 
-def check_operator_problem(cc, shape, seed=7):
+def check_operator_problem(cc, shape, seed=7, plain=True):
     """conv_relu_forward and the three conv_relu_backward_* operators (accumulating), the plain
     operators (conv_forward, conv_backward_x, conv_backward_kb) and the three plain backward
-    operators as one call (conv_backward_xkb), against the oracle."""
+    operators as one call (conv_backward_xkb), against the oracle.  ``plain=False`` leaves the
+    one-by-one plain operators out (problems of several GB, where each oracle call takes
+    seconds): the kernels are the same template with the mask compiled out."""
     ref = make_problem(shape, torch.float32, seed=seed)
-    dev = make_problem(shape, torch.float32, device="cuda", seed=seed)
+    dev = problem_on(ref, "cuda")
     d = ref["d"]
     oracle.conv_relu_forward(ref["x"], ref["k"], ref["bias"], ref["y"], d)
     cc.conv_relu_forward(dev["x"], dev["k"], dev["bias"], dev["y"], d)
@@ -41,9 +43,23 @@ def check_operator_problem(cc, shape, seed=7):
     assert torch.equal(dev["gy"].cpu(), ref["gy"]), "conv_relu_backward_x wrote outside grad_input"
     assert rel_err(got_gk, want_gk) <= 1e-4, "conv_relu_backward_k"
     assert bias_close(got_gb, want_gb, ref["gy"] * (ref["y"] > 0)), "conv_relu_backward_bias"
+    if not plain:
+        # the fused pass on the same data: grad_input accumulates once more, no mask
+        want_gk, want_gb = torch.zeros_like(ref["k"]), torch.zeros_like(ref["bias"])
+        oracle.conv_backward_x(ref["gy"], ref["k"], ref["gx"], d)
+        oracle.conv_backward_k(ref["gy"], ref["x"], want_gk, d)
+        oracle.conv_backward_bias(ref["gy"], want_gb)
+        got_gk, got_gb = torch.zeros_like(dev["k"]), torch.zeros_like(dev["bias"])
+        cc.conv_backward_xkb(dev["gy"], dev["x"], dev["k"], dev["gx"], got_gk, got_gb, d)
+        torch.cuda.synchronize()
+        assert rel_err(dev["gstack"], ref["gstack"]) <= 1e-4, "conv_backward_xkb grad_input"
+        assert rel_err(got_gk, want_gk) <= 1e-4, "conv_backward_xkb grad_kernel"
+        assert bias_close(got_gb, want_gb, ref["gy"]), "conv_backward_xkb grad_bias"
+        return
+    del ref, dev
     # the plain (no-ReLU) operators one by one
     ref3 = make_problem(shape, torch.float32, seed=seed + 2)
-    dev3 = make_problem(shape, torch.float32, device="cuda", seed=seed + 2)
+    dev3 = problem_on(ref3, "cuda")
     want_gk, want_gb = torch.zeros_like(ref3["k"]), torch.zeros_like(ref3["bias"])
     oracle.conv_forward(ref3["x"], ref3["k"], ref3["bias"], ref3["y"], d)
     oracle.conv_backward_x(ref3["gy"], ref3["k"], ref3["gx"], d)
@@ -59,8 +75,9 @@ def check_operator_problem(cc, shape, seed=7):
     assert rel_err(got_gk, want_gk) <= 1e-4, "conv_backward_kb grad_kernel"
     assert bias_close(got_gb, want_gb, ref3["gy"]), "conv_backward_kb grad_bias"
     # the three plain operators in one call
+    del ref3, dev3
     ref2 = make_problem(shape, torch.float32, seed=seed + 1)
-    dev2 = make_problem(shape, torch.float32, device="cuda", seed=seed + 1)
+    dev2 = problem_on(ref2, "cuda")
     want_gk, want_gb = torch.zeros_like(ref2["k"]), torch.zeros_like(ref2["bias"])
     oracle.conv_backward_x(ref2["gy"], ref2["k"], ref2["gx"], d)
     oracle.conv_backward_k(ref2["gy"], ref2["x"], want_gk, d)

@@ -166,3 +166,25 @@ def test_loss_gradient_scales_with_the_incoming_gradient():
     (3 * model.loss).backward()
     for name, g in _grads(model).items():
         assert rel_err(g, 3 * once[name]) <= 1e-6, name
+
+
+def test_a_hook_anywhere_in_the_net_switches_the_fused_loss_off():
+    # forward hooks see a module's own call: with one on any module of `net` (here the outer
+    # Sequential and the LogSoftmax, which the fused node never calls) the modules run one by one
+    from msd_pytorch_amd import MSDSegmentationModel
+    torch.manual_seed(6)
+    model = MSDSegmentationModel(1, 3, 4, 1)
+    model.msd.final_layer.linear.weight.data.normal_(0, 0.2)
+    x, t = torch.rand(1, 1, 24, 64), torch.randint(0, 3, (1, 1, 24, 64))
+    plain = model.forward(x, t)
+    assert type(model.loss.grad_fn).__name__ == "MSDNetLossFunctionBackward"
+    for module in (model.net, model.net[1][1], model.scale_in):
+        seen = []
+        handle = module.register_forward_hook(lambda m, i, o: seen.append(tuple(o.shape)))
+        hooked = model.forward(x, t)
+        handle.remove()
+        assert seen == [(1, 1 if module is model.scale_in else 3, 24, 64)]
+        assert type(model.loss.grad_fn).__name__ != "MSDNetLossFunctionBackward"
+        assert abs(hooked - plain) <= 1e-5 * abs(plain)
+    model.forward(x, t)
+    assert type(model.loss.grad_fn).__name__ == "MSDNetLossFunctionBackward"

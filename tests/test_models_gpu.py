@@ -506,6 +506,57 @@ def test_train_with_a_recorded_step_follows_the_eager_loop():
     assert abs(recorded.get_loss() - eager.get_loss()) <= 1e-5 * max(1.0, abs(eager.get_loss()))
 
 
+def test_train_with_a_recorded_step_leaves_gpu_resident_batches_alone():
+    # batches that are on the GPU already (set_input / set_target keep such tensors as they
+    # are): the recorded step copies later batches into buffers of its own, not into the
+    # caller's first batch; a smaller last batch gets a recorded step of its own, once
+    from msd_pytorch_amd import MSDRegressionModel
+    import warnings
+    size = (32, 64)
+    torch.manual_seed(23)
+    batches = [(torch.randn(2, 1, *size).cuda(), torch.randn(2, 1, *size).cuda()) for _ in range(3)]
+    batches.append((torch.randn(1, 1, *size).cuda(), torch.randn(1, 1, *size).cuda()))
+    copies = [(a.clone(), b.clone()) for a, b in batches]
+    models = []
+    for _ in range(2):
+        torch.manual_seed(22)
+        m = MSDRegressionModel(1, 1, depth=4, width=1, dilations=[1, 2, 3])
+        m.msd.final_layer.linear.weight.data.normal_(0, 0.2)
+        models.append(m)
+    eager, recorded = models
+    eager.train(batches, 2)
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")          # no stream-mismatch warning from the capture
+        recorded.train(batches, 2, graph=True)
+    torch.cuda.synchronize()
+    for (a, b), (a0, b0) in zip(batches, copies):
+        assert torch.equal(a, a0) and torch.equal(b, b0)
+    for a, b in zip(recorded.msd.parameters(), eager.msd.parameters()):
+        assert rel_err(a.detach(), b.detach()) <= 1e-5
+
+
+def test_train_checks_gpu_resident_labels_without_waiting_per_batch():
+    # labels on the GPU: train() validates them on the device and raises once per epoch,
+    # where set_target (msd_segmentation_model.py:105-119) raises at once
+    from msd_pytorch_amd import MSDSegmentationModel
+    torch.manual_seed(24)
+    model = MSDSegmentationModel(1, 3, depth=3, width=1, dilations=[1, 2])
+    x = torch.randn(1, 1, 24, 64).cuda()
+    good = torch.randint(0, 3, (1, 1, 24, 64)).cuda()
+    model.train([(x, good)] * 3, 1)
+    assert model.get_loss() == model.get_loss()
+    with pytest.raises(ValueError):
+        model.set_target(good + 1)
+    with pytest.raises(ValueError):
+        model.train([(x, good), (x, good + 1)], 1)
+    with pytest.raises(ValueError):
+        model.train([(x, good * -1)], 1)
+    model.train([(x, good)], 1)                 # the verdict of a failed epoch is not carried over
+    # host tensors are still checked on the host, batch by batch
+    with pytest.raises(ValueError):
+        model.train([(x.cpu(), (good + 1).cpu())], 1)
+
+
 def test_regression_state_dict_keys():
     # key layout of the reference's checkpoints (msd_regression_model.py:76, msd_block.py:170-179)
     from msd_pytorch_amd import MSDRegressionModel

@@ -95,6 +95,57 @@ def test_static_scratch_matches_the_oracle_and_the_python_wrapper():
         assert rel_err(gk, want_gk) <= 1e-4 and rel_err(gb, want_gb) <= 1e-4
 
 
+def _static_call(lib, p, gk, gb):
+    from msd_pytorch_amd import _native
+    x, y, gy = p["x"], p["y"], p["gy"]
+    ndim = x.dim() - 2
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    rc = lib.msd_conv_relu_backward_kb_static(
+        _native.MSD_F32, ndim, x.shape[0], x.shape[1], y.shape[1], _i64(x.shape[2:]), p["d"], _ptr(y), _i64(y.stride()),
+        _ptr(gy), _i64(gy.stride()), _ptr(x), _i64(x.stride()), _ptr(gk), _ptr(gb), stream)
+    assert rc == 0, lib.msd_last_error().decode()
+
+
+@pytest.mark.parametrize("shape", [(1, 19, 1, (48, 512), 3), (1, 9, 1, (10, 12, 128), 2)])
+def test_static_scratch_allocates_nothing_and_can_be_captured(shape):
+    # what the entry point is for: no device memory is taken by a call (free bytes of the
+    # device unchanged across raw C-ABI calls), and once the first call on the device has
+    # looked the buffer's address up, a call can be recorded into a HIP graph; every replay
+    # (with eager work between the replays) gives the bits of the eager call
+    from msd_pytorch_amd import _native
+    from msd_pytorch_amd import msd_custom_convolutions as cc
+    lib = _native.load()
+    p = make_problem(shape, torch.float32, device="cuda", seed=41)
+    cc.conv_relu_forward(p["x"], p["k"], p["bias"], p["y"], p["d"])
+    gk, gb = torch.zeros_like(p["k"]), torch.zeros_like(p["bias"])
+    _static_call(lib, p, gk, gb)                       # first call: looks the address up
+    torch.cuda.synchronize()
+    want_gk, want_gb = gk.clone(), gb.clone()
+    free_before = torch.cuda.mem_get_info()[0]
+    for _ in range(3):
+        gk.zero_(), gb.zero_()
+        _static_call(lib, p, gk, gb)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
+    assert torch.equal(gk, want_gk) and torch.equal(gb, want_gb)
+
+    graph = torch.cuda.CUDAGraph()
+    gk.zero_(), gb.zero_()
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph):
+        _static_call(lib, p, gk, gb)                   # accumulates into gk, gb
+    for replay in range(3):
+        gk.zero_(), gb.zero_()
+        other = make_problem((1, 3, 1, (20, 64), 1), torch.float32, device="cuda", seed=50 + replay)
+        cc.conv_relu_forward(other["x"], other["k"], other["bias"], other["y"], other["d"])
+        ogk, ogb = torch.zeros_like(other["k"]), torch.zeros_like(other["bias"])
+        _static_call(lib, other, ogk, ogb)             # eager work through the same buffer in between
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(gk, want_gk) and torch.equal(gb, want_gb), replay
+
+
 def test_static_scratch_rejects_what_does_not_fit():
     from msd_pytorch_amd import _native
     from msd_pytorch_amd import msd_custom_convolutions as cc
