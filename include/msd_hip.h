@@ -79,7 +79,9 @@ int msd_set_kernel_path(int path);
  * numbered by residue class), "fwd.lattice3d" (24, 33 or 44: rows z x y of a 3D forward tile;
  * 0: chosen by the library), "block.pair" (0/1: the backward pass of a 2D block of one-channel
  * layers takes its layers two or three at a time), "block.triple" (0: never three at a time,
- * n > 0: three where the layers share at least n channels; 32 by default).
+ * n > 0: three where the layers share at least n channels; 32 by default), "final.tiled" (0/1:
+ * msd_final_forward_loss reads the stack once, through LDS tiles, where it can: fp32, up to 128
+ * input and 4 output channels).
  * Unknown keys return MSD_ERR_INVALID.
  */
 int msd_set_tuning(const char *key, int value);

@@ -11,9 +11,13 @@
 //             so the result does not depend on scheduling.
 // Output channels are handled in groups of at most MAXO per launch.
 #include "msd_kernels.h"
+#include "msd_rows.h"
 
+#include <algorithm>
 #include <initializer_list>
+#include <mutex>
 #include <utility>
+#include <vector>
 
 namespace msd {
 
@@ -288,6 +292,239 @@ __global__ __launch_bounds__(kFinalThreads) void final_forward_loss_kernel(
     }
 }
 
+// The same pass for up to 128 input channels with the stack read ONCE (fp32): a workgroup of
+// eight waves owns a tile of 64 * V voxels; lane l of every wave stands for the same V voxels
+// and wave w takes the channels c % 8 == w.  First walk: each wave loads its channels of the
+// tile (all requests issued before the first use), adds its share of the outputs and leaves
+// the values in LDS; the eight partial outputs meet in LDS, every wave forms the loss
+// gradient g of its lanes' voxels; second walk: each wave takes its channels back from LDS
+// and adds g * x to per-lane running sums, which live in registers over all tiles of the
+// workgroup (tile t, t + grid, ...) and are reduced over the lanes once at the end: one row
+// of partial sums per workgroup.  Same columns of `part` as the kernel above.
+constexpr int kTiledWaves = 8;
+constexpr int kTiledThreads = kTiledWaves * kWave;
+constexpr int kTiledMaxChannels = 128;
+
+template <int V, int MAXO, int KIND, int CC>
+__global__ __launch_bounds__(kTiledThreads, 4) void final_forward_loss_tiled(
+    int64_t nvec, int tiles_per_image, int total_tiles, int C, int c_out, const float *__restrict__ x, int64_t xsb,
+    int64_t xsc, const float *__restrict__ w, const float *__restrict__ bias, const void *__restrict__ target,
+    int64_t tsb, int64_t tsc, float *__restrict__ out, int64_t osb, int64_t osc, float *__restrict__ gout, int64_t gsb,
+    int64_t gsc, float inv_n, int want_sums, float *__restrict__ part, int64_t rows)
+{
+    extern __shared__ float lds_tile[];
+    // weights and bias are read-only for the whole kernel: addressed as constant memory they
+    // are wave-uniform scalar loads (as plain global loads next to the stores of the loop they
+    // would each take a vector register)
+    typedef const __attribute__((address_space(4))) float *const_floats_t;
+    const const_floats_t wk = (const_floats_t)(uintptr_t)w;
+    const const_floats_t bk = (const_floats_t)(uintptr_t)bias;
+    constexpr int TV = kWave * V;                             // voxels of a tile
+    float *red = lds_tile + (size_t)C * TV;                   // [wave][o][e][lane]; then g as [o][e][lane]
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
+    float sw[MAXO][CC], sb[MAXO], lsum = 0.f;
+#pragma unroll
+    for (int o = 0; o < MAXO; o++) {
+        sb[o] = 0.f;
+#pragma unroll
+        for (int cc = 0; cc < CC; cc++) sw[o][cc] = 0.f;
+    }
+    // this wave's weights: w[o][c] for c = cc * 8 + wave (zero past the last channel)
+    for (int tile = blockIdx.x; tile < total_tiles; tile += gridDim.x) {
+        // new values as far as the compiler knows: the weights (scalar loads) and the channels'
+        // offsets are formed again per tile instead of being kept, and spilled, over the loop
+        asm volatile("" : "+s"(xsc), "+s"(C));
+        const int b = tile / tiles_per_image;
+        const int64_t i = (int64_t)(tile - b * tiles_per_image) * kWave + lane;
+        const bool active = i < nvec;
+        const int64_t ic = active ? i : nvec - 1;             // lanes past the end work on a valid voxel, contribute zeros
+        // a uniform base per channel plus one 32-bit lane offset: no address registers per request
+        const uint64_t xbase = reinterpret_cast<uint64_t>(x + (int64_t)b * xsb);
+        const uint32_t xoff = (uint32_t)(ic * V) * 4u;
+        float acc[MAXO][V];
+#pragma unroll
+        for (int o = 0; o < MAXO; o++)
+#pragma unroll
+            for (int e = 0; e < V; e++) acc[o][e] = 0.f;
+        // channels in groups of G requests (16 registers), all of a group issued before its first use
+        constexpr int G = CC < 16 / V ? CC : 16 / V;
+#pragma unroll
+        for (int c0 = 0; c0 < CC; c0 += G) {
+            float v[G][V];
+#pragma unroll
+            for (int j = 0; j < G; j++)
+                load_global_vec<V>(xbase + (uint64_t)((int64_t)min((c0 + j) * kTiledWaves + wave, C - 1) * xsc * 4), xoff,
+                                   v[j]);
+#pragma unroll
+            for (int j = 0; j < G; j++) {
+                const int c = (c0 + j) * kTiledWaves + wave;  // uniform
+                if (c < C) {
+#pragma unroll
+                    for (int o = 0; o < MAXO; o++) {
+                        const float wv = wk[(int64_t)min(o, c_out - 1) * C + c];
+#pragma unroll
+                        for (int e = 0; e < V; e++) acc[o][e] += wv * v[j][e];
+                    }
+                    store_elems<float, V>(lds_tile + (size_t)c * TV + lane * V, v[j]);
+                }
+            }
+        }
+#pragma unroll
+        for (int o = 0; o < MAXO; o++)
+#pragma unroll
+            for (int e = 0; e < V; e++) red[((wave * MAXO + o) * V + e) * kWave + lane] = acc[o][e];
+        __syncthreads();
+        // the eight partial outputs in a fixed order (a loop that stays a loop: unrolled, all
+        // 8 * MAXO * V values would be requested at once and held in registers)
+#pragma unroll
+        for (int o = 0; o < MAXO; o++)
+#pragma unroll
+            for (int e = 0; e < V; e++) acc[o][e] = red[(o * V + e) * kWave + lane];
+#pragma unroll 1
+        for (int q = 1; q < kTiledWaves; q++) {
+            const float *rq = red + (size_t)q * MAXO * V * kWave + lane;
+#pragma unroll
+            for (int o = 0; o < MAXO; o++)
+#pragma unroll
+                for (int e = 0; e < V; e++) acc[o][e] += rq[(o * V + e) * kWave];
+        }
+        float g[MAXO][V];
+        float tile_loss = 0.f;
+        if constexpr (KIND == 2) {
+            // the softmax is the expensive part: wave q forms it for element q of every lane's
+            // voxels only, and the waves exchange the results through LDS below
+            const int64_t *lab = static_cast<const int64_t *>(target) + (int64_t)b * tsb + ic * V;
+#pragma unroll
+            for (int e = 0; e < V; e++) {
+                if (wave != e) continue;                      // uniform
+                float m = acc[0][e] + (bias ? bk[0] : 0.f);
+#pragma unroll
+                for (int o = 0; o < MAXO; o++) {
+                    acc[o][e] += bias && o < c_out ? bk[o] : 0.f;
+                    if (o < c_out) m = acc[o][e] > m ? acc[o][e] : m;
+                }
+                float se = 0.f;
+#pragma unroll
+                for (int o = 0; o < MAXO; o++)
+                    if (o < c_out) se += exp(acc[o][e] - m);
+                const float lse = m + log(se);
+                const int64_t t = lab[e];
+#pragma unroll
+                for (int o = 0; o < MAXO; o++) {
+                    acc[o][e] -= lse;                         // log-probability
+                    const float pr = o < c_out ? exp(acc[o][e]) : 0.f;
+                    g[o][e] = active && o < c_out ? (pr - (t == o ? 1.f : 0.f)) * inv_n : 0.f;
+                    if (active && t == o) tile_loss -= acc[o][e];
+                }
+            }
+        } else {
+#pragma unroll
+            for (int o = 0; o < MAXO; o++) {
+                const bool keep = active && o < c_out;
+                float t[V];
+                load_elems<float, V>(static_cast<const float *>(target) + (int64_t)b * tsb +
+                                         (int64_t)min(o, c_out - 1) * tsc + ic * V, t);
+                const float bv = bias && o < c_out ? bk[o] : 0.f;
+#pragma unroll
+                for (int e = 0; e < V; e++) {
+                    acc[o][e] += bv;
+                    const float diff = acc[o][e] - t[e];
+                    if (KIND == 0) {
+                        g[o][e] = keep ? 2.f * diff * inv_n : 0.f;
+                        tile_loss += keep ? diff * diff : 0.f;
+                    } else {
+                        g[o][e] = keep ? (diff > 0.f ? inv_n : (diff < 0.f ? -inv_n : 0.f)) : 0.f;
+                        tile_loss += keep ? (diff < 0.f ? -diff : diff) : 0.f;
+                    }
+                }
+            }
+        }
+        if constexpr (KIND == 2) {
+            // wave e wrote nothing of the other elements: log-probabilities and g through LDS
+            __syncthreads();                                  // all waves have read the partial outputs
+            float *gs = red, *ls = red + MAXO * V * kWave;    // [o][e][lane] each
+#pragma unroll
+            for (int e = 0; e < V; e++)
+                if (wave == e) {
+#pragma unroll
+                    for (int o = 0; o < MAXO; o++) {
+                        gs[(o * V + e) * kWave + lane] = g[o][e];
+                        ls[(o * V + e) * kWave + lane] = acc[o][e];
+                    }
+                }
+            __syncthreads();
+#pragma unroll
+            for (int o = 0; o < MAXO; o++)
+#pragma unroll
+                for (int e = 0; e < V; e++) {
+                    g[o][e] = gs[(o * V + e) * kWave + lane];
+                    acc[o][e] = ls[(o * V + e) * kWave + lane];
+                }
+            // (tile_loss: each of the waves 0 .. V - 1 holds the terms of its element)
+        }
+        if (wave == 0 || (KIND == 2 && wave < V)) lsum += tile_loss * inv_n;
+        if (wave == 0) {                                      // uniform: one wave writes the outputs
+            if (active) {
+#pragma unroll
+                for (int o = 0; o < MAXO; o++) {
+                    if (o >= c_out) break;
+                    store_elems<float, V>(out + (int64_t)b * osb + (int64_t)o * osc + i * V, acc[o]);
+                    store_elems<float, V>(gout + (int64_t)b * gsb + (int64_t)o * gsc + i * V, g[o]);
+                }
+            }
+#pragma unroll
+            for (int o = 0; o < MAXO; o++)
+#pragma unroll
+                for (int e = 0; e < V; e++) sb[o] += g[o][e];
+        }
+        if (want_sums) {                                      // uniform
+#pragma unroll
+            for (int cc = 0; cc < CC; cc++) {
+                const int c = cc * kTiledWaves + wave;
+                if (c < C) {
+                    float xv[V];
+                    load_elems<float, V>(lds_tile + (size_t)c * TV + lane * V, xv);   // what this wave stored itself
+#pragma unroll
+                    for (int o = 0; o < MAXO; o++)
+#pragma unroll
+                        for (int e = 0; e < V; e++) sw[o][cc] += g[o][e] * xv[e];
+                }
+            }
+        }
+        __syncthreads();                                      // `red` is rewritten by the next tile
+    }
+    const int64_t row = blockIdx.x;
+    {
+        // the loss terms of the waves that hold some (wave 0; NLL: waves 0 .. V - 1), in order
+        lsum = wave_sum(lsum);
+        if (lane == 0) red[wave] = lsum;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            float t = red[0];
+            if constexpr (KIND == 2)
+                for (int q = 1; q < V; q++) t += red[q];
+            part[((int64_t)c_out * C + c_out) * rows + row] = t;
+        }
+    }
+    if (!want_sums) return;
+    if (wave == 0) {
+#pragma unroll
+        for (int o = 0; o < MAXO; o++) {
+            const float s = wave_sum(sb[o]);
+            if (lane == 0 && o < c_out) part[((int64_t)c_out * C + o) * rows + row] = s;
+        }
+    }
+#pragma unroll
+    for (int cc = 0; cc < CC; cc++) {
+        const int c = cc * kTiledWaves + wave;
+#pragma unroll
+        for (int o = 0; o < MAXO; o++) {
+            const float s = wave_sum(sw[o][cc]);
+            if (lane == 0 && o < c_out && c < C) part[((int64_t)o * C + c) * rows + row] = s;
+        }
+    }
+}
+
 // One workgroup per column: thread t adds rows t, t + 256, ... in order, a fixed shuffle tree
 // adds the lanes of each wave and the four wave sums are added in order.
 // Columns [0, nw) go to gw, [nw, nw + nb) to gb, a last one (if any) to `loss`.
@@ -409,12 +646,153 @@ hipError_t final_backward(int64_t batch, int c_in, int c_out, int64_t nvox, cons
     return hipGetLastError();
 }
 
+namespace {
+
+// Kernels that ask for more than 64 KB of LDS need the attribute set once per kernel and
+// device (it stays); later launches, also ones recorded into a graph, go without the call.
+hipError_t allow_large_lds(const void *kernel, size_t bytes)
+{
+    static std::mutex mutex;
+    static std::vector<std::pair<const void *, int>> done;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    std::lock_guard<std::mutex> lock(mutex);
+    for (const auto &d : done)
+        if (d.first == kernel && d.second == dev) return hipSuccess;
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e == hipSuccess) done.emplace_back(kernel, dev);
+    return e;
+}
+
+constexpr size_t kTiledLdsLimit = 80 * 1024;     // two workgroups share the 160 KB of a CU
+
+template <int V, int MAXO, int KIND, int CC>
+hipError_t launch_tiled(int64_t batch, int c_in, int c_out, int64_t nvox, const float *x, int64_t xsb, int64_t xsc,
+                        const float *w, const float *bias, const void *target, int64_t tsb, int64_t tsc, float *out,
+                        int64_t osb, int64_t osc, float *gout, int64_t gsb, int64_t gsc, float inv_n, int want,
+                        float *ws, int64_t *rows, hipStream_t s)
+{
+    const int64_t nvec = nvox / V;
+    const int64_t tiles_per_image = (nvec + kWave - 1) / kWave;
+    const int64_t total = tiles_per_image * batch;
+    if (total > INT32_MAX) return hipErrorInvalidConfiguration;
+    const size_t lds = ((size_t)c_in * kWave * V + (size_t)kTiledWaves * MAXO * V * kWave) * sizeof(float);
+    const void *fn = reinterpret_cast<const void *>(&final_forward_loss_tiled<V, MAXO, KIND, CC>);
+    if (lds > 64 * 1024) {
+        const hipError_t e = allow_large_lds(fn, kTiledLdsLimit);
+        if (e != hipSuccess) return e;
+    }
+    const int grid = (int)std::min<int64_t>(total, 512);      // two workgroups per CU, each walks its tiles
+    *rows = grid;
+    hipLaunchKernelGGL((final_forward_loss_tiled<V, MAXO, KIND, CC>), dim3(grid), dim3(kTiledThreads), lds, s, nvec,
+                       (int)tiles_per_image, (int)total, c_in, c_out, x, xsb, xsc, w, bias, target, tsb, tsc, out, osb,
+                       osc, gout, gsb, gsc, inv_n, want, ws, (int64_t)grid);
+    return hipGetLastError();
+}
+
+// V-wide accesses at multiples of V are aligned in every view given.
+inline bool vec_aligned(int v, int64_t nvox, std::initializer_list<std::pair<const void *, std::pair<int64_t, int64_t>>> views)
+{
+    if (nvox % v != 0) return false;
+    for (const auto &vw : views) {
+        if (!vw.first) continue;
+        if (reinterpret_cast<uintptr_t>(vw.first) % (v * sizeof(float)) != 0 || vw.second.first % v != 0 ||
+            vw.second.second % v != 0)
+            return false;
+    }
+    return true;
+}
+
+// The tiled kernel where it applies (fp32, up to 128 input and 4 output channels, a tile that
+// fits the LDS); *handled says whether it was launched.
+hipError_t final_forward_loss_tiled_try(int kind, int64_t batch, int c_in, int c_out, int64_t nvox, const float *x,
+                                        int64_t xsb, int64_t xsc, const float *w, const float *bias,
+                                        const void *target, int64_t tsb, int64_t tsc, float *out, int64_t osb,
+                                        int64_t osc, float *gout, int64_t gsb, int64_t gsc, float inv_n, int want,
+                                        float *ws, int64_t *rows, hipStream_t s, bool *handled)
+{
+    *handled = false;
+    if (c_in > kTiledMaxChannels || c_out > 4 || !knob(kKnobFinalTiled, 1)) return hipSuccess;
+    const int mo = c_out > 2 ? 4 : (c_out > 1 ? 2 : 1);
+    int v = 0;
+    for (int cand = 4; cand >= 1; cand /= 2) {
+        const bool aligned =
+            kind == 2 ? vec_aligned(cand, nvox, {{x, {xsb, xsc}}, {out, {osb, osc}}, {gout, {gsb, gsc}}})
+                      : vec_aligned(cand, nvox, {{x, {xsb, xsc}}, {out, {osb, osc}}, {gout, {gsb, gsc}}, {target, {tsb, tsc}}});
+        const size_t lds = ((size_t)c_in * kWave * cand + (size_t)kTiledWaves * mo * cand * kWave) * sizeof(float);
+        if (aligned && lds <= kTiledLdsLimit && (cand < 4 || c_in <= 64)) {
+            v = cand;
+            break;
+        }
+    }
+    if (v == 0) return hipSuccess;
+    const bool wide = c_in > 64;                              // sixteen channels per wave instead of eight
+#define MSD_TILED(VV, OO, KK, CCC)                                                                                    \
+    return (*handled = true, launch_tiled<VV, OO, KK, CCC>(batch, c_in, c_out, nvox, x, xsb, xsc, w, bias, target, tsb, \
+                                                          tsc, out, osb, osc, gout, gsb, gsc, inv_n, want, ws, rows, s))
+#define MSD_TILED_C(VV, OO, KK)                                  \
+    do {                                                         \
+        if (VV == 4 || !wide) MSD_TILED(VV, OO, KK, 8);          \
+        if constexpr (VV != 4) MSD_TILED(VV, OO, KK, 16);        \
+    } while (0)
+#define MSD_TILED_K(VV, OO)                                                                     \
+    do {                                                                                        \
+        if (kind == 0) MSD_TILED_C(VV, OO, 0); else if (kind == 1) MSD_TILED_C(VV, OO, 1); else MSD_TILED_C(VV, OO, 2); \
+    } while (0)
+#define MSD_TILED_O(VV)                                                                         \
+    do {                                                                                        \
+        if (mo == 4) MSD_TILED_K(VV, 4); else if (mo == 2) MSD_TILED_K(VV, 2); else MSD_TILED_K(VV, 1); \
+    } while (0)
+    if (v == 4) MSD_TILED_O(4); else if (v == 2) MSD_TILED_O(2); else MSD_TILED_O(1);
+#undef MSD_TILED_O
+#undef MSD_TILED_K
+#undef MSD_TILED_C
+#undef MSD_TILED
+    return hipSuccess;
+}
+
+template <typename T> struct TiledLoss {
+    static hipError_t run(int, int64_t, int, int, int64_t, const T *, int64_t, int64_t, const T *, const T *,
+                          const void *, int64_t, int64_t, T *, int64_t, int64_t, T *, int64_t, int64_t, T, int, T *,
+                          int64_t *, hipStream_t, bool *handled)
+    {
+        *handled = false;
+        return hipSuccess;
+    }
+};
+template <> struct TiledLoss<float> {
+    template <typename... A> static hipError_t run(A... a) { return final_forward_loss_tiled_try(a...); }
+};
+
+}  // namespace
+
 template <typename T>
 hipError_t final_forward_loss(int kind, int64_t batch, int c_in, int c_out, int64_t nvox, const T *x, int64_t xsb,
                               int64_t xsc, const T *w, const T *bias, const void *target, int64_t tsb, int64_t tsc,
                               T *out, int64_t osb, int64_t osc, T *gout, int64_t gsb, int64_t gsc, T *gw, T *gb,
                               T *loss, T *ws, hipStream_t s)
 {
+    {
+        const int64_t terms = kind == 2 ? batch * nvox : batch * nvox * (int64_t)c_out;
+        bool handled = false;
+        int64_t rows = 0;
+        const hipError_t e = TiledLoss<T>::run(kind, batch, c_in, c_out, nvox, x, xsb, xsc, w, bias, target, tsb, tsc, out,
+                                               osb, osc, gout, gsb, gsc, T(1) / T(terms), (int)(gw || gb), ws, &rows, s,
+                                               &handled);
+        if (e != hipSuccess) return e;
+        if (handled) {
+            const int64_t nw = (int64_t)c_out * c_in;
+            if (gw || gb) {
+                hipLaunchKernelGGL(final_reduce_kernel<T>, dim3((unsigned)(nw + c_out + 1)), dim3(256), 0, s, ws, rows,
+                                   nw, (int64_t)c_out, gw, gb, loss);
+            } else {
+                hipLaunchKernelGGL(final_reduce_kernel<T>, dim3(1), dim3(256), 0, s, ws + (nw + c_out) * rows, rows,
+                                   (int64_t)0, (int64_t)0, (T *)nullptr, (T *)nullptr, loss);
+            }
+            return hipGetLastError();
+        }
+    }
     // labels are one int64 per voxel: no vector width to match
     const int V = kind == 2 ? final_vec<T>(nvox, {{x, {xsb, xsc}}, {out, {osb, osc}}, {gout, {gsb, gsc}}})
                             : final_vec<T>(nvox, {{x, {xsb, xsc}}, {out, {osb, osc}}, {gout, {gsb, gsc}},

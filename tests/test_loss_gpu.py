@@ -42,6 +42,13 @@ CASES = [
     (2, 6, 4, (3, 5, 7)),
     (1, 5, 8, (9, 11)),
     (1, 9, 2, (8, 12)),
+    # more than 64 and more than 128 input channels (sixteen channels per wave; the walk-twice kernel),
+    # several tiles per workgroup and a ragged last tile
+    (1, 70, 4, (24, 50)),
+    (2, 101, 4, (130, 258)),
+    (1, 51, 1, (12, 40, 64)),
+    (1, 130, 2, (16, 20)),
+    (1, 33, 3, (700, 1030)),
 ]
 
 
@@ -49,6 +56,41 @@ CASES = [
 @pytest.mark.parametrize("kind", ["mse", "l1", "nll"])
 @pytest.mark.parametrize("batch,c_in,c_out,spatial", CASES)
 def test_fused_loss_matches_torch(batch, c_in, c_out, spatial, kind, dtype):
+    if dtype == torch.float64 and batch * c_in * spatial[0] * spatial[1] > 1 << 20:
+        pytest.skip("the large cases are there for the fp32 kernels")
+    check_fused_loss(batch, c_in, c_out, spatial, kind, dtype)
+
+
+@pytest.mark.parametrize("kind", ["mse", "l1", "nll"])
+@pytest.mark.parametrize("batch,c_in,c_out,spatial", CASES)
+def test_fused_loss_walking_the_stack_twice_matches_torch(batch, c_in, c_out, spatial, kind):
+    # the kernel that reads the stack twice (what fp64, wide stacks and more than four output
+    # channels take), forced for the shapes the single-read kernel would take
+    from msd_pytorch_amd import _native
+    lib = _native.load()
+    assert lib.msd_set_tuning(b"final.tiled", 0) == 0
+    try:
+        check_fused_loss(batch, c_in, c_out, spatial, kind, torch.float32)
+    finally:
+        lib.msd_set_tuning(b"final.tiled", -1)
+
+
+def test_fused_loss_is_reproducible():
+    from msd_pytorch_amd import msd_custom_convolutions as cc
+    gen = torch.Generator().manual_seed(9)
+    x = torch.randn(2, 90, 64, 130, generator=gen).cuda()
+    w, b = (torch.randn(4, 90, generator=gen) * 0.2).cuda(), torch.randn(4, generator=gen).cuda()
+    t = torch.randint(0, 4, (2, 64, 130), generator=gen).cuda()
+    runs = []
+    for _ in range(3):
+        gw, gb = torch.empty(4, 90, device="cuda"), torch.empty(4, device="cuda")
+        out, loss, g = cc.final_forward_loss(x, w, b, "nll", t, gw, gb)
+        runs.append((out.clone(), loss.clone(), g.clone(), gw, gb))
+    for r in runs[1:]:
+        assert all(torch.equal(a, b) for a, b in zip(r, runs[0]))
+
+
+def check_fused_loss(batch, c_in, c_out, spatial, kind, dtype):
     from msd_pytorch_amd import msd_custom_convolutions as cc
     gen = torch.Generator().manual_seed(c_in * 100 + c_out)
     # the input is a channel slice of a larger stack, as the dense block hands it over
