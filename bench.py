@@ -37,7 +37,7 @@ FAMILIES = {"forward": ("fwd_lattice",), "backward_xkb": ("bwd_rows_fused", "bwd
 SECOND_PASS = ("reduce_columns",)
 
 
-def profiled_traffic(name):
+def profiled_traffic(name, split3d=False):
     """HBM-side bytes per pass of the network for each kernel class, read from the committed
     rocprofv3 summary of this workload (profiles/bench_workload_<name>_*.txt, block "HBM-side
     bytes per pass": FETCH_SIZE + WRITE_SIZE per dispatch, scaled by what the same counters
@@ -70,7 +70,12 @@ def profiled_traffic(name):
             else:
                 block = None
     out = {}
-    for cls, fams in FAMILIES.items():
+    families = dict(FAMILIES)
+    if split3d:
+        # the weight gradients of two layers per pass are instances of the fused kernel's family
+        families["backward_kb"] = ("bwd_rows_fused", "reduce_columns", "bwdk_rows", "bwdk_mfma")
+        families["backward_xkb"] = ()
+    for cls, fams in families.items():
         found = [per_family[f] for f in fams if f in per_family]
         if found:
             main = [dispatches[f] for f in fams if f in dispatches and f not in SECOND_PASS]
@@ -128,7 +133,7 @@ def make_model(name, torch):
     return model
 
 
-def algorithmic_work(name, fused, paired=False, triple_from=32):
+def algorithmic_work(name, fused, paired=False, triple_from=32, kpairs=False):
     """Per-step algorithmic bytes and flops of each kernel class, fp32, per layer with C input
     and w output channels over N voxels and K = 9 or 27 taps:
     bytes: forward (C + w) N 4, backward_x (2C + 2w) N 4, backward_k+bias (C + 2w) N 4, the fused
@@ -144,6 +149,10 @@ def algorithmic_work(name, fused, paired=False, triple_from=32):
     one pass over the c channels below all n layers with the layers as its n output channels,
     (3c + 2n) N 4 bytes: what that algorithm has to move, a half to a third of the per-layer
     figure.  The per-layer figure is returned as well, under "backward_xkb_per_layer".
+    `kpairs`: the library runs a 3D block of width 1 as a chain of backward_x launches with the
+    weight and bias gradients of two layers per pass over x beside it (layers depth-1 and depth-2,
+    ... down to 1 and 0; an odd lowest layer alone): a pair reads the C input channels of its
+    upper layer once and two output gradients, (C + 4) N 4 bytes.
     Returns (bytes per class, flops per class, voxels per step)."""
     kind, ndim, c_in, c_out, depth, width, batch, spatial, adam = WORKLOADS[name]
     n = batch
@@ -181,8 +190,13 @@ def algorithmic_work(name, fused, paired=False, triple_from=32):
         if i > 0:
             nbytes["backward_x"] += (2 * C + 2 * width) * n * 4 + wts
             flops["backward_x"] += op
-        nbytes["backward_kb"] += (C + 2 * width) * n * 4 + wts
         flops["backward_kb"] += op
+        if kpairs and (depth - 1 - i) % 2 == 1:
+            continue                          # the lower layer of a pair: counted with the upper one
+        if kpairs and i > 0:
+            nbytes["backward_kb"] += (C + 4 * width) * n * 4 + 2 * wts
+        else:
+            nbytes["backward_kb"] += (C + 2 * width) * n * 4 + wts
     return nbytes, flops, n
 
 
@@ -311,7 +325,13 @@ def measure(name, args, lib, torch, steps=None, warmup=None, cpu=True):
         paired = ndim == 2 and width == 1 and tuned.get("block.pair") != "0" and tuned.get("block.fuse") != "0"
         triple = int(tuned.get("block.triple", -1))
         triple_from = None if triple == 0 else (32 if triple < 0 else triple)
-        bytes_per_step, flops_per_step, _ = algorithmic_work(name, totals["backward_xkb"][1] > 0, paired, triple_from)
+        # 3D blocks of width 1 may run as a chain of backward_x launches with the weight gradients
+        # two layers per pass on a second stream (block.split3d); the instrumented repeat runs both
+        # on one stream, so the classes' times add up to more than the step's backward pass
+        split3d = ndim == 3 and width == 1 and totals["backward_xkb"][1] == 0 and \
+            0 < totals["backward_kb"][1] // args.steps < depth
+        bytes_per_step, flops_per_step, _ = algorithmic_work(name, totals["backward_xkb"][1] > 0, paired, triple_from,
+                                                             kpairs=split3d)
         kernels = {}
         for cls, (ms, launches) in totals.items():
             if launches == 0:
@@ -335,7 +355,10 @@ def measure(name, args, lib, torch, steps=None, warmup=None, cpu=True):
         dominant = max(kernels, key=lambda c: kernels[c]["ms_per_step"])
         dom = kernels[dominant]
         # the committed counter figures describe the library's default launch shapes
-        traffic, source = ({}, None) if args.tune else profiled_traffic(name)
+        traffic, source = ({}, None) if args.tune else profiled_traffic(name, split3d)
+        if split3d:
+            result["config"]["backward"] = ("chain of backward_x launches; weight gradients two layers per pass on a "
+                                            "second stream (kernel classes timed on one stream)")
         per_launch, profiled_calls = traffic.get(dominant, (None, None))
         stale = per_launch is not None and profiled_calls is not None and profiled_calls != dom["calls_per_step"]
         if stale:

@@ -81,7 +81,10 @@ int msd_set_kernel_path(int path);
  * layers takes its layers two or three at a time), "block.triple" (0: never three at a time,
  * n > 0: three where the layers share at least n channels; 32 by default), "final.tiled" (0/1:
  * msd_final_forward_loss reads the stack once, through LDS tiles, where it can: fp32, up to 128
- * input and 4 output channels).
+ * input and 4 output channels), "block.split3d" (the backward pass of a 3D block of one-channel
+ * layers; 1: a chain of backward_x launches on the caller's stream and the weight gradients, two
+ * layers per pass, on a second stream that is forked from and joined to the caller's inside the
+ * call; 2: the same launches on the caller's stream alone; 0: one fused launch per layer).
  * Unknown keys return MSD_ERR_INVALID.
  */
 int msd_set_tuning(const char *key, int value);

@@ -17,9 +17,9 @@ const char *const kKnobNames[kKnobCount] = {
     "xcd_remap", "bwdk.vec2d", "bwdk.vec3d", "bwdk.blocks",
     "fwd.vec2d", "fwd.vec3d", "fwd.split", "fwd.rows2d", "bwdk.rows", "block.fuse",
     "block.defer", "bwdk.interleave", "block.snake", "fwd.class3d", "fwd.lattice3d",
-    "block.pair", "block.triple", "final.tiled",
+    "block.pair", "block.triple", "final.tiled", "block.split3d",
 };
-static_assert(kKnobFinalTiled + 1 == kKnobCount, "one name per knob, in the order of the enum");
+static_assert(kKnobBlockSplit3d + 1 == kKnobCount, "one name per knob, in the order of the enum");
 int g_knobs[kKnobCount];
 // every knob starts at "library default"
 const bool g_knobs_ready = [] {
@@ -721,6 +721,11 @@ int64_t block_layer_workspace(int dtype, int ndim, int64_t batch, int64_t c_in, 
         if (widths[i] <= 0) return -1;
         int64_t n = msd_workspace_bytes(dtype, ndim, batch, total, widths[i], spatial);
         if (n < 0) return -1;
+        if (ndim == 3 && i + 1 < depth && widths[i + 1] == 1 && widths[i] == 1) {
+            // 3D: the weight gradients of this layer and the one above it in one pass
+            const int64_t nup = msd_workspace_bytes(dtype, ndim, batch, total + 1, 2, spatial);
+            n = nup > n ? nup : n;
+        }
         for (int up = 1; up < msd::kMaxLayerGroup; up++) {
             // this layer and the one or two above it may run as the output channels of one pass
             if (ndim != 2 || i + up >= depth || widths[i + up] != 1 || widths[i] != 1) break;
@@ -884,6 +889,7 @@ int block_group_fused(const char *fn, const BlockArgs &a, int i, int n, int64_t 
         const int bottom = i - j + 1;             // output channel 0 of this launch
         int dmax = 0;
         st.group.n = j;
+        st.group.lowest_channels = 0;
         for (int q = 0; q < j; q++) {
             st.group.dil[q] = (int)a.dilations[bottom + q];
             dmax = st.group.dil[q] > dmax ? st.group.dil[q] : dmax;
@@ -933,6 +939,177 @@ int block_group_fused(const char *fn, const BlockArgs &a, int i, int n, int64_t 
                                                 shared ? (float *)gb_lowest : nullptr, (float *)ws, s, job, grp);
         if (e != hipSuccess) return hip_fail(fn, e);
         if (job) pending->taken(region);
+    }
+    *done = true;
+    return MSD_OK;
+}
+
+// ---------------------------------------------------------------------------
+// 3D blocks of one-channel layers: the reverse loop as two streams of work.
+//
+// Only the input gradient makes the reverse loop a chain (layer i's masked output gradient
+// is complete once every layer above has added its share to that channel); the weight and
+// bias gradients of a layer need nothing but that output gradient and the activations.
+// So the chain runs as lean backward_x launches (the gather and a read-modify-write stream
+// over grad_input, nothing else in registers), and the weight gradients follow on a second
+// stream, two layers per pass over x on the matrix cores (fast_backward_k_pair_3d): x is
+// read once per two layers, and the chain's launches and the matrix-core launches fill each
+// other's gaps.  The second stream is forked from the caller's with an event per pair and
+// joined to it before the call returns, so the caller sees one stream's semantics (also
+// while its stream is being captured into a graph, once the stream and events exist).
+// ---------------------------------------------------------------------------
+struct SideStream {
+    hipStream_t s = nullptr;
+    std::vector<hipEvent_t> events;               // fork events, used in turn; the last one joins
+    size_t next = 0;
+};
+constexpr int kSideEvents = 32;
+std::mutex g_side_mutex;
+SideStream g_side[64];
+
+// The current device's second stream, made on first use (default priority); nullptr when it
+// cannot be made (the caller then runs everything on its own stream).
+SideStream *side_stream()
+{
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+    std::lock_guard<std::mutex> lock(g_side_mutex);
+    SideStream &side = g_side[dev];
+    if (side.s) return &side;
+    hipStream_t s = nullptr;
+    if (hipStreamCreateWithFlags(&s, hipStreamNonBlocking) != hipSuccess) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    std::vector<hipEvent_t> events;
+    for (int i = 0; i < kSideEvents + 1; i++) {
+        hipEvent_t e;
+        if (hipEventCreateWithFlags(&e, hipEventDisableTiming) != hipSuccess) {
+            (void)hipGetLastError();
+            for (hipEvent_t made : events) (void)hipEventDestroy(made);
+            (void)hipStreamDestroy(s);
+            return nullptr;
+        }
+        events.push_back(e);
+    }
+    side.s = s;
+    side.events = events;
+    return &side;
+}
+
+// *done is false (and nothing was launched) when the block is not one this path takes.
+int block_backward_split3d(const char *fn, const BlockArgs &a, int64_t c_in, const void *stack,
+                           const int64_t *stack_strides, void *grads, const int64_t *grads_strides,
+                           const void *const *weights, void *const *grad_weights, void *grad_bias, bool need_input_grad,
+                           void *workspace, int64_t workspace_bytes, hipStream_t main, DeferredReductions *pending,
+                           bool *done)
+{
+    *done = false;
+    // By default for volumes of up to 4 M voxels: the two streams gain what the launches' ramps
+    // and tails leave idle (about 15 to 30 microseconds per launch), the separate kernels lose a
+    // share of the fused pass's time that grows with the volume (128^3, depth 50: 7.7 against
+    // 8.2 ms; 256^3, depth 30: 28.9 against 25.0 ms).
+    int64_t voxels = a.batch;
+    for (int d = 0; d < a.ndim; d++) voxels *= a.spatial[d];
+    const int mode = msd::knob(msd::kKnobBlockSplit3d, voxels <= ((int64_t)1 << 22) ? 1 : 0);
+    if (mode == 0 || a.dtype != MSD_F32 || a.ndim != 3 || g_kernel_path != 0 || !grad_bias || a.depth < 2 ||
+        !msd::knob(msd::kKnobBlockFuse, 1))
+        return MSD_OK;
+    for (int i = 0; i < a.depth; i++)
+        if (a.widths[i] != 1 || !grad_weights[i]) return MSD_OK;
+    msd::View<const float> x;
+    msd::View<float> gx;
+    MSD_TRY(make_view(fn, "input", a.ndim, stack, stack_strides, &x));
+    MSD_TRY(make_view(fn, "grad_input", a.ndim, grads, grads_strides, &gx));
+    const bool same_layout = x.sb == gx.sb && x.sc == gx.sc && x.sz == gx.sz && x.sy == gx.sy &&
+                             reinterpret_cast<uintptr_t>(x.p) % 16 == reinterpret_cast<uintptr_t>(gx.p) % 16;
+    if (!same_layout) return MSD_OK;
+    // every launch of the plan must be one the specialised kernels take
+    struct Pair {
+        msd::Geom g;
+        msd::LayerGroup group;
+        msd::View<const float> gy;
+    };
+    std::vector<Pair> pairs(a.depth);             // pairs[l]: layers (l + 1, l), l the lower one
+    std::vector<msd::Geom> chain(a.depth);
+    for (int i = a.depth - 1; i >= 0; i--) {
+        const int64_t first = c_in + i;           // channels layer i reads; its output is channel `first`
+        MSD_TRY(make_geom(fn, a.dtype, a.ndim, a.batch, first, 1, a.spatial, (int)a.dilations[i], true, &chain[i]));
+        const msd::View<const float> gy{gx.p + first * gx.sc, gx.sb, gx.sc, gx.sz, gx.sy, gx.sx};
+        if ((i > 0 || need_input_grad) && !msd::fast_backward_x_supported(chain[i], false, gy, gy, gx)) return MSD_OK;
+        const bool lower = (a.depth - 1 - i) % 2 == 1;
+        if (lower) {
+            Pair &p = pairs[i];
+            const int du = (int)a.dilations[i + 1], dl = (int)a.dilations[i];
+            MSD_TRY(make_geom(fn, a.dtype, a.ndim, a.batch, first + 1, 2, a.spatial, du > dl ? du : dl, true, &p.g));
+            p.group.n = 2;
+            p.group.dil[0] = dl;
+            p.group.dil[1] = du;
+            p.group.dil[2] = 0;
+            p.group.k_up[0] = p.group.k_up[1] = nullptr;
+            p.group.gk_up[0] = (float *)grad_weights[i + 1];
+            p.group.gk_up[1] = nullptr;
+            p.group.lowest_channels = (int)first;
+            p.gy = gy;                            // channels first (layer i) and first + 1 (layer i + 1)
+            if (!msd::fast_backward_k_pair_supported_3d(p.g, p.gy, x)) return MSD_OK;
+            MSD_TRY(check_workspace(fn, p.g, sizeof(float), workspace, workspace_bytes));
+        }
+    }
+    // a profiled run keeps to one stream: its per-class event pairs time one stream's work
+    SideStream *side = (mode == 1 && !g_profile.on) ? side_stream() : nullptr;
+    const hipStream_t ks = side ? side->s : main;
+    pending->s = ks;
+    auto fork = [&]() -> int {                    // what follows on the second stream waits for the chain so far
+        if (!side) return MSD_OK;
+        hipEvent_t e = side->events[side->next];
+        side->next = (side->next + 1) % kSideEvents;
+        hipError_t err = hipEventRecord(e, main);
+        if (err == hipSuccess) err = hipStreamWaitEvent(side->s, e, 0);
+        return err == hipSuccess ? MSD_OK : hip_fail(fn, err);
+    };
+    bool masked = false;
+    for (int i = a.depth - 1; i >= 0; i--) {
+        const int64_t first = c_in + i;
+        const char *out_i = (const char *)stack + first * stack_strides[1] * a.elem;
+        char *gout_i = (char *)grads + first * grads_strides[1] * a.elem;
+        if (!masked)
+            MSD_TRY(msd_relu_mask_gradient(a.dtype, a.ndim, a.batch, 1, a.spatial, out_i, stack_strides, gout_i,
+                                           grads_strides, main));
+        masked = false;
+        // the output gradients of layer i (and of layer i + 1) are final here
+        const bool lower = (a.depth - 1 - i) % 2 == 1;
+        if (lower) {
+            Pair &p = pairs[i];
+            MSD_TRY(fork());
+            const int64_t region = partial_region_floats(a.ndim, p.g.C, 2);
+            msd::ReduceJob *job = nullptr;
+            MSD_TRY(pending->next(fn, region, &job));
+            ProfileScope scope(2, ks);
+            p.g.reverse = msd::knob(msd::kKnobBlockSnake, 1) && (i & 2);
+            const hipError_t e = msd::fast_backward_k_pair_3d(p.g, p.gy, x, (float *)grad_weights[i],
+                                                              (float *)grad_bias + i, (float *)workspace, ks, job,
+                                                              &p.group);
+            if (e != hipSuccess) return hip_fail(fn, e);
+            if (job) pending->taken(region);
+        } else if (i == 0) {
+            // an odd layer is left at the bottom: the single-layer operator
+            MSD_TRY(fork());
+            MSD_TRY(backward_kb("conv_backward_kb", false, true, a.dtype, a.ndim, a.batch, first, 1, a.spatial,
+                                (int)a.dilations[i], nullptr, nullptr, gout_i, grads_strides, stack, stack_strides,
+                                grad_weights[i], (char *)grad_bias + i * a.elem, workspace, workspace_bytes, ks));
+        }
+        if (i > 0 || need_input_grad)
+            MSD_TRY(backward_x("conv_backward_x", false, a.dtype, a.ndim, a.batch, first, 1, a.spatial,
+                               (int)a.dilations[i], nullptr, nullptr, gout_i, grads_strides, weights[i], grads,
+                               grads_strides, main, i > 0 ? (int)(first - 1) : (int)first, i > 0 ? stack : nullptr,
+                               stack_strides, &masked));
+    }
+    MSD_TRY(pending->flush(fn));
+    if (side) {
+        hipEvent_t join = side->events[kSideEvents];
+        hipError_t err = hipEventRecord(join, side->s);
+        if (err == hipSuccess) err = hipStreamWaitEvent(main, join, 0);
+        if (err != hipSuccess) return hip_fail(fn, err);
     }
     *done = true;
     return MSD_OK;
@@ -1003,6 +1180,14 @@ int msd_block_backward(int dtype, int ndim, int64_t batch, int64_t c_in, int dep
     if (workspace && layer_ws >= 0 && workspace_bytes > layer_ws && msd::knob(msd::kKnobBlockDefer, 1)) {
         pending.base = (float *)((char *)workspace + layer_ws);
         pending.capacity = (workspace_bytes - layer_ws) / (int64_t)sizeof(float);
+    }
+    {
+        bool done = false;
+        MSD_TRY(block_backward_split3d(fn, a, c_in, stack, stack_strides, grads, grads_strides, weights, grad_weights,
+                                       grad_bias, need_input_grad != 0, workspace, workspace_bytes, (hipStream_t)stream,
+                                       &pending, &done));
+        if (done) return MSD_OK;
+        pending.s = (hipStream_t)stream;
     }
     bool masked = false;   // the mask of the current layer was already applied by the previous backward_x
     int groups_done = 0;

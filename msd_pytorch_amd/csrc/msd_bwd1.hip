@@ -227,7 +227,7 @@ hipError_t fast_backward_one_channel_2d(const Geom &g, const View<const float> &
     if (e != hipSuccess) return e;
     const int64_t nk = (int64_t)g.Wd * bwd1::K;
     const ReduceJob job{part, gk, nullptr, nk, nk, wgs, {group ? group->gk_up[0] : nullptr, nullptr},
-                        group ? (int64_t)bwd1::K : nk};
+                        group ? (int64_t)bwd1::K : nk, group ? (int64_t)bwd1::K : nk};
     if (defer) {
         *defer = job;
         return hipSuccess;

@@ -20,4 +20,15 @@ hipError_t fast_backward_xkb_3d(const Geom &g, const View<const float> &gy, cons
     }
 }
 
+bool fast_backward_k_pair_supported_3d(const Geom &g, const View<const float> &gy, const View<const float> &x)
+{
+    return bwdxk::k_pair_supported_3d(g, gy, x);
+}
+
+hipError_t fast_backward_k_pair_3d(const Geom &g, const View<const float> &gy, const View<const float> &x, float *gk,
+                                   float *gb, float *ws, hipStream_t s, ReduceJob *defer, const LayerGroup *group)
+{
+    return bwdxk::k_pair_3d(g, gy, x, gk, gb, ws, s, defer, group);
+}
+
 }  // namespace msd

@@ -98,7 +98,7 @@ struct Args {
 // The waves' tiles share the LDS of the staged rows (two outputs at four voxels per lane: the
 // tiles alone are 79 KB; three outputs, or 3D at two voxels per lane: 59 KB).
 template <int NDIM, int V, int WOUT>
-constexpr bool tiles_over_staging() { return (NDIM == 2 && ((V == 4 && WOUT == 2) || WOUT == 3)) || (NDIM == 3 && V == 2); }
+constexpr bool tiles_over_staging() { return (NDIM == 2 && ((V == 4 && WOUT == 2) || WOUT == 3)) || (NDIM == 3 && (V == 2 || WOUT >= 2)); }
 
 // Workgroups (of four waves) that are resident per CU.  The 3D kernel with one voxel per lane
 // (pipeline stages of 16 voxels, arguments read again per tile, row arithmetic on the scalar
@@ -130,7 +130,11 @@ template <int NDIM, int V, int NCB, int WOUT, bool LONG> constexpr int pipeline_
 // BIG (LONG instances only): the 64-bit channel bases and the loads from any address; without it
 // a LONG instance only cuts rows into segments and addresses like the plain one (whole groups of
 // four voxels, stacks below 2^30 values), which saves a fifth of a stage's instructions.
-template <int NDIM, int V, int NCB, int WOUT, bool LONG, bool BIG = LONG>
+// KONLY: the weight and bias gradients alone (no grad_input update: no weights, no loads or
+// stores of grad_input); what is left is the gather, the A tile and a stream over x on the
+// matrix cores.  The dense block uses it for two 3D layers per pass, beside a chain of
+// backward_x launches on another stream.
+template <int NDIM, int V, int NCB, int WOUT, bool LONG, bool BIG = LONG, bool KONLY = false>
 __global__ __launch_bounds__(kThreads, (resident_per_cu<NDIM, V, NCB, WOUT, LONG>()))
 void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *__restrict__ xp,
                     float *__restrict__ gxp, const float *__restrict__ actp, const float *__restrict__ kw,
@@ -238,6 +242,62 @@ void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *_
     // allocation around them grows (3D, up to 32 channels per chunk: 142-150 -> 108-116 VGPRs,
     // which is what lets a fourth workgroup share the CU).  The 2D instances with two output
     // channels gain 1 % (245 -> 220 VGPRs at most); those with one are 2 % slower that way.
+    // One step of the workgroup's walk: from the tile at (grp, seg, gi, b, y0, z0, row, y, z) to its next one.
+    auto advance = [&](const Args &a, int &grp, int &seg, int &gi, int &b, int &y0, int &z0, int &row, int &y, int &z) {
+        const Geom &g = a.g;
+        const RowTeams &rt = a.rt;
+        grp += a.group_step;
+        int carry = 0;
+        if constexpr (SEG) {
+            seg += a.step.seg;
+            if (seg >= a.sg.segs) {
+                seg -= a.sg.segs;
+                carry = 1;
+            }
+        }
+        gi += a.step.gi + carry;
+        b += a.step.b;
+        if constexpr (NDIM == 3) {
+            y0 += a.step.y + (carry ? a.step.carry_y : 0);
+            z0 += a.step.z + (carry ? a.step.carry_z : 0);
+        }
+        if (gi >= a.ngroups) {                    // into the next batch item
+            gi -= a.ngroups;
+            b++;
+            if constexpr (NDIM == 3) {
+                y0 -= a.step.wrap_y;
+                z0 -= a.step.wrap_z;
+            }
+        }
+        row = gi * rt.rpw + team;
+        if constexpr (NDIM == 3) {
+            while (y0 >= g.H) {
+                y0 -= g.H;
+                z0++;
+            }
+            while (y0 < 0) {
+                y0 += g.H;
+                z0--;
+            }
+            y = y0 + team;
+            z = z0;
+            while (y >= g.H) {
+                y -= g.H;
+                z++;
+            }
+        } else {
+            y = row;
+        }
+    };
+    // KONLY: the first source rows of the tile to come (msd_rows.h: request_source_rows)
+    float pre[KONLY ? WOUT : 1][KONLY ? NPQ : 1][V];
+    if constexpr (KONLY) {
+        if (grp < a.total_groups) {
+            const bool ok0 = row < rt.nrows;
+            const View<const float> gyv{gyp, a.gy.sb, a.gy.sc, a.gy.sz, a.gy.sy, 1};
+            request_source_rows<NDIM, WOUT, V>(g, gyv, b, ok0 ? z : g.D - 1, ok0 ? y : g.H - 1, lane, pre, a.up);
+        }
+    }
     constexpr bool RELOAD = NDIM == 3 || WOUT == 2;
     typedef const __attribute__((address_space(4))) int *kernarg_words_t;
     kernarg_words_t kernarg = (kernarg_words_t)__builtin_amdgcn_kernarg_segment_ptr();
@@ -310,10 +370,12 @@ void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *_
                 for (int j = 0; j < NSS; j++)
                     load_global_vec<4>(xbase, 4u * (xch + (uint32_t)min(kx + 16 * (h * NSS + j), g.W - 4)), kk[j]);
             }
+            if constexpr (!KONLY) {
 #pragma unroll
-            for (int j = 0; j < NCS; j++) {
-                const int ci = max(min(c0 + cb * kChanBlock + h * NCS + j, cx_end - 1), 0);
-                load_global_vec<V>(channel_base(gbase, ci), goff, gg[j]);
+                for (int j = 0; j < NCS; j++) {
+                    const int ci = max(min(c0 + cb * kChanBlock + h * NCS + j, cx_end - 1), 0);
+                    load_global_vec<V>(channel_base(gbase, ci), goff, gg[j]);
+                }
             }
         };
         // XPAIR: x of the pair of 16-voxel groups 2 * pair, 2 * pair + 1 (one cache line per channel) ...
@@ -336,7 +398,18 @@ void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *_
         // block of 16 channels that stage `s` of the walk belongs to
         auto block_of = [&](int s) { return g.reverse ? ncb - 1 - s / H : s / H; };
         // issued ahead of the gather so the latencies overlap (a tile has at least H >= NSETS stages)
-        if constexpr (XPAIR) {
+        // KONLY: a ring of four pairs of 16-voxel groups, each requested three pairs ahead of its use
+        // (two waves per SIMD and nothing but matrix instructions between request and use)
+        float xring[KONLY ? 4 : 1][2][4];
+        const int npairs = 2 * ncb;
+        auto pair_block = [&](int p) {
+            const int blk = min(p, npairs - 1) / 2;
+            return g.reverse ? ncb - 1 - blk : blk;
+        };
+        if constexpr (KONLY) {
+#pragma unroll
+            for (int q = 0; q < 3; q++) load_x2(pair_block(q), min(q, npairs - 1) % 2, xring[q]);
+        } else if constexpr (XPAIR) {
             load_x2(block_of(0), 0, xpa);
             load_g(block_of(0), 0, gs_[0]);
         } else {
@@ -350,7 +423,10 @@ void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *_
             const View<const float> none{nullptr, 0, 0, 0, 0, 0};
             const View<const float> gyv{gyp, a.gy.sb, a.gy.sc, a.gy.sz, a.gy.sy, 1};
             float own[WOUT][NPQ][V];
-            if (segmented) {
+            if constexpr (KONLY) {
+                // the rows were asked for during the tile before (before the loop for the first)
+                finish_source_rows<NDIM, WOUT, V>(g, rt, gyv, b, zc, yc, lane, act, S, pre, own, a.up);
+            } else if (segmented) {
                 if constexpr (SEG)
                     stage_source_segment<NDIM, WOUT, V>(g, rt, a.sg, gyv, b, zc, yc, xs, lane, rowok, S, own, a.up);
             } else {
@@ -425,6 +501,16 @@ void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *_
                 for (int co = 0; co < WOUT; co++)
 #pragma unroll
                     for (int i = 0; i < V; i++) bsum[co] += tv[co * K + K / 2][i];
+            }
+        }
+        if constexpr (KONLY) {
+            // the next tile's source rows, in flight during this tile's channel loop
+            int ngrp = grp, nseg = seg, ngi = gi, nb = b, ny0 = y0, nz0 = z0, nrow = row, ny = y, nz = z;
+            advance(a, ngrp, nseg, ngi, nb, ny0, nz0, nrow, ny, nz);
+            if (ti + 1 < a_.tiles_per_wg && ngrp < a.total_groups) {
+                const bool nok = nrow < rt.nrows;
+                const View<const float> gyv{gyp, a.gy.sb, a.gy.sc, a.gy.sz, a.gy.sy, 1};
+                request_source_rows<NDIM, WOUT, V>(g, gyv, nb, nok ? nz : g.D - 1, nok ? ny : g.H - 1, lane, pre, a.up);
             }
         }
         // the tile is private to the wave and LDS executes a wave's accesses in order: only
@@ -539,7 +625,40 @@ void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *_
         // ---- channel loop: blocks of 16 channels, H stages each, NSETS stages per iteration (all of
         // one block); the loads of stage s + NSETS - 1 are issued before the arithmetic of stage s
         const int nst = ncb * H;                  // a multiple of NSETS
-        if constexpr (XPAIR) {
+        if constexpr (KONLY) {
+            // x alone: four pairs (two blocks of 16 channels) per iteration of the loop
+            static_assert(XPAIR, "the weight-gradient-only instances are the 3D ones with one voxel per lane");
+#pragma unroll 1
+            for (int p0 = 0; p0 < npairs; p0 += 4) {
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    const int p = p0 + u;
+                    // (past the last pair the last one is asked for again: never used, a cache hit)
+                    load_x2(pair_block(p + 3), min(p + 3, npairs - 1) % 2, xring[(u + 3) % 4]);
+                    if (p < npairs) {             // uniform
+                        const int cb = pair_block(p);
+                        if (u % 2 == 0) {
+#pragma unroll
+                            for (int tg = 0; tg < TG; tg++)
+#pragma unroll
+                                for (int c = 0; c < NCH; c++) acc[tg][c] = mfma4{0.f, 0.f, 0.f, 0.f};
+                        }
+                        stage_k(cb, 2 * (u % 2), reinterpret_cast<float (&)[NSS][4]>(xring[u][0]));
+                        stage_k(cb, 2 * (u % 2) + 1, reinterpret_cast<float (&)[NSS][4]>(xring[u][1]));
+                        if (u % 2 == 1) {
+#pragma unroll
+                            for (int q = 0; q < NCB; q++)
+                                if (q == cb) {
+#pragma unroll
+                                    for (int tg = 0; tg < TG; tg++)
+#pragma unroll
+                                        for (int c = 0; c < NCH; c++) D[q][tg] += acc[tg][c];
+                                }
+                        }
+                    }
+                }
+            }
+        } else if constexpr (XPAIR) {
             // one block of 16 channels (four stages) per iteration.  Every load is issued a stage
             // or more ahead of its use and none sits behind a test (loads retire in order, and the
             // compiler sizes each wait for the path with the fewest loads behind the one it needs):
@@ -622,48 +741,7 @@ void bwd_rows_fused(const Args a_, const float *__restrict__ gyp, const float *_
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         if constexpr (ALIAS) __syncthreads();     // the next tile's staged rows overwrite every wave's tile
         // next tile (all of this is uniform)
-        grp += a.group_step;
-        int carry = 0;
-        if constexpr (SEG) {
-            seg += a.step.seg;
-            if (seg >= a.sg.segs) {
-                seg -= a.sg.segs;
-                carry = 1;
-            }
-        }
-        gi += a.step.gi + carry;
-        b += a.step.b;
-        if constexpr (NDIM == 3) {
-            y0 += a.step.y + (carry ? a.step.carry_y : 0);
-            z0 += a.step.z + (carry ? a.step.carry_z : 0);
-        }
-        if (gi >= a.ngroups) {                    // into the next batch item
-            gi -= a.ngroups;
-            b++;
-            if constexpr (NDIM == 3) {
-                y0 -= a.step.wrap_y;
-                z0 -= a.step.wrap_z;
-            }
-        }
-        row = gi * rt.rpw + team;
-        if constexpr (NDIM == 3) {
-            while (y0 >= g.H) {
-                y0 -= g.H;
-                z0++;
-            }
-            while (y0 < 0) {
-                y0 += g.H;
-                z0--;
-            }
-            y = y0 + team;
-            z = z0;
-            while (y >= g.H) {
-                y -= g.H;
-                z++;
-            }
-        } else {
-            y = row;
-        }
+        advance(a, grp, seg, gi, b, y0, z0, row, y, z);
     }
 
     // D[cb][tg][v] = sum for tap tg*16 + 4*mk + v, channel c0 + cb*16 + mj.  Add the waves in LDS.
@@ -753,7 +831,7 @@ bool fits(const Geom &g, int V, const View<const float> &gy, const View<const fl
     const size_t kr = (size_t)g.Wd * Taps<NDIM>::K + 1;
     const size_t staged = (size_t)rt.rpw * g.Wd * RowTaps<NDIM>::NPQ * (V * rt.lpr + sg.halo) * 4;
     const size_t tiles = (size_t)kWaves * kr * (kWave * V + 4) * 4;
-    const bool over = (NDIM == 2 && ((V == 4 && g.Wd == 2) || g.Wd == 3)) || (NDIM == 3 && V == 2);   // tiles_over_staging()
+    const bool over = (NDIM == 2 && ((V == 4 && g.Wd == 2) || g.Wd == 3)) || (NDIM == 3 && (V == 2 || g.Wd >= 2));   // tiles_over_staging()
     if ((over ? std::max(staged, tiles) : staged + tiles) > (over ? kMaxLdsBytesAsked : kMaxLdsBytes)) return false;
     return rows_aligned(gy, g.W, V) && rows_aligned(gx, g.W, V);
 }
@@ -774,7 +852,7 @@ int choose_vec(const Geom &g, int vmax, const View<const float> &gy, const View<
 
 // `group`: the output channels are layers of a dense block (g.dil is then the largest of their
 // dilations, which is what the row segments' halo is sized for).
-template <int NDIM, int V, int NCB, int WOUT, bool LONG, bool BIG = LONG>
+template <int NDIM, int V, int NCB, int WOUT, bool LONG, bool BIG = LONG, bool KONLY = false>
 hipError_t launch(const Geom &g, const View<const float> &gy, const View<const float> &x, const float *k,
                   const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws, hipStream_t s,
                   ReduceJob *defer, const LayerGroup *group)
@@ -841,7 +919,7 @@ hipError_t launch(const Geom &g, const View<const float> &gy, const View<const f
         if (e != hipSuccess) return e;
         const uint64_t bit = dev >= 0 && dev < 64 ? (uint64_t)1 << dev : 0;
         if (!(asked.load(std::memory_order_acquire) & bit)) {
-            e = hipFuncSetAttribute(reinterpret_cast<const void *>(&bwd_rows_fused<NDIM, V, NCB, WOUT, LONG, BIG>),
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(&bwd_rows_fused<NDIM, V, NCB, WOUT, LONG, BIG, KONLY>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLdsBytesAsked);
             if (e != hipSuccess) return e;
             asked.fetch_or(bit, std::memory_order_release);
@@ -850,7 +928,7 @@ hipError_t launch(const Geom &g, const View<const float> &gy, const View<const f
     // the weights of the upper output channels follow those of the first, or are other layers'
     const float *k1 = group ? group->k_up[0] : k + (int64_t)g.C * K;
     const float *k2 = group ? group->k_up[1] : k + (int64_t)2 * g.C * K;
-    hipLaunchKernelGGL((bwd_rows_fused<NDIM, V, NCB, WOUT, LONG, BIG>), dim3(rows, 1, chunks), dim3(a.rt.lpr * a.rt.rpw), lds, s, a,
+    hipLaunchKernelGGL((bwd_rows_fused<NDIM, V, NCB, WOUT, LONG, BIG, KONLY>), dim3(rows, 1, chunks), dim3(a.rt.lpr * a.rt.rpw), lds, s, a,
                        gy.p, x.p, gx.p, actp, k, k1, k2, part);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
@@ -858,8 +936,11 @@ hipError_t launch(const Geom &g, const View<const float> &gy, const View<const f
     const int64_t ncols = nk + (a.want_bias ? WOUT : 0);
     // a group's columns: [0, split) of the partial sums go to gk, the next `split` ones to the
     // second layer's weight gradient, the rest to the third's
+    // (KONLY pairs run over one channel more than the lower layer has: its columns of that
+    // channel are dropped by the reduction)
+    const int64_t per_layer = group ? (int64_t)g.C * K : nk;
     const ReduceJob job{part, gk, gb, nk, ncols, rows, {group ? group->gk_up[0] : nullptr, group ? group->gk_up[1] : nullptr},
-                        group ? (int64_t)g.C * K : nk};
+                        per_layer, group && group->lowest_channels > 0 ? (int64_t)group->lowest_channels * K : per_layer};
     if (defer) {
         *defer = job;
         return hipSuccess;
@@ -998,6 +1079,28 @@ hipError_t xkb_nd(const Geom &g, const View<const float> &gy, const View<const f
     }
     if (v == 1) return pick_ncb<NDIM, 1, 1, LONG>(g, gy, x, k, gx, pm, gk, gb, ws, s, defer, nullptr);
     return hipErrorInvalidConfiguration;
+}
+
+// Weight and bias gradients of two 3D layers of a dense block in one pass over the input
+// channels of the upper one (plain instances, one voxel per lane, up to 64 channels per chunk
+// of the grid): whether the shapes fit, and the launch.
+inline bool k_pair_supported_3d(const Geom &g, const View<const float> &gy, const View<const float> &x)
+{
+    if (g.ndim != 3 || g.Wd != 2 || x.sx != 1 || gy.sx != 1) return false;
+    if (!small_strides(g, gy) || !small_strides(g, x) || !x_offsets_fit(g, x, false)) return false;
+    const View<float> none{const_cast<float *>(gy.p), gy.sb, gy.sc, gy.sz, gy.sy, gy.sx};   // (grad_input is not touched)
+    return fits<3>(g, 1, gy, x, none, false);
+}
+
+inline hipError_t k_pair_3d(const Geom &g, const View<const float> &gy, const View<const float> &x, float *gk, float *gb,
+                            float *ws, hipStream_t s, ReduceJob *defer, const LayerGroup *group)
+{
+    const View<float> none{nullptr, 0, 0, 0, 0, 1};
+    const PostMask pm{g.C, {nullptr, 0, 0, 0, 0, 0}};
+    const int need = (g.C + kChanBlock - 1) / kChanBlock;
+    if (need <= 1) return launch<3, 1, 1, 2, false, false, true>(g, gy, x, nullptr, none, pm, gk, gb, ws, s, defer, group);
+    if (need <= 2) return launch<3, 1, 2, 2, false, false, true>(g, gy, x, nullptr, none, pm, gk, gb, ws, s, defer, group);
+    return launch<3, 1, 4, 2, false, false, true>(g, gy, x, nullptr, none, pm, gk, gb, ws, s, defer, group);
 }
 
 }  // namespace bwdxk

@@ -346,8 +346,9 @@ __global__ __launch_bounds__(kTiledThreads, 4) void final_forward_loss_tiled(
         for (int o = 0; o < MAXO; o++)
 #pragma unroll
             for (int e = 0; e < V; e++) acc[o][e] = 0.f;
-        // channels in groups of G requests (16 registers), all of a group issued before its first use
-        constexpr int G = CC < 16 / V ? CC : 16 / V;
+        // channels in groups of G requests, all of a group issued before its first use: all of
+        // the wave's channels at once where the running sums leave the registers for it
+        constexpr int G = MAXO * CC + V * CC < 96 ? CC : (CC < 24 / V ? CC : 24 / V);
 #pragma unroll
         for (int c0 = 0; c0 < CC; c0 += G) {
             float v[G][V];

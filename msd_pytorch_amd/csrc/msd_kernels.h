@@ -61,7 +61,7 @@ enum Knob {
     kKnobXcdRemap, kKnobBwdkVec2d, kKnobBwdkVec3d, kKnobBwdkBlocks,
     kKnobFwdVec2d, kKnobFwdVec3d, kKnobFwdSplit, kKnobFwdRows2d, kKnobBwdkRows, kKnobBlockFuse,
     kKnobBlockDefer, kKnobBwdkInterleave, kKnobBlockSnake, kKnobFwdClass3d, kKnobFwdLattice3d,
-    kKnobBlockPair, kKnobBlockTriple, kKnobFinalTiled,
+    kKnobBlockPair, kKnobBlockTriple, kKnobFinalTiled, kKnobBlockSplit3d,
     kKnobCount
 };
 int knob(Knob k, int dflt);
@@ -152,6 +152,7 @@ struct ReduceJob {
     float *gk_up[2];  // columns [split, 2 split) and [2 split, nk) go here instead of to gk (the weight
                       // gradients of a second and a third layer)
     int64_t split;    // nk where there is no other destination
+    int64_t valid0;   // columns [valid0, split) are dropped (= split: none)
 };
 // Two or three layers of a dense block as the output channels of one fused backward pass over
 // the input channels they share: output channel 0 is the lowest layer (dilation dil[0], the
@@ -164,6 +165,7 @@ struct LayerGroup {
     int dil[kMaxLayerGroup];
     const float *k_up[kMaxLayerGroup - 1];
     float *gk_up[kMaxLayerGroup - 1];
+    int lowest_channels;   // > 0: the lowest layer has only this many of the pass's input channels
 };
 constexpr int kReduceBatch = 16;
 // One launch for up to kReduceBatch pending reductions; every column is added in the same
@@ -184,6 +186,14 @@ hipError_t fast_backward_xkb_2d(const Geom &g, const View<const float> &gy, cons
 hipError_t fast_backward_xkb_3d(const Geom &g, const View<const float> &gy, const View<const float> &x, const float *k,
                                 const View<float> &gx, const PostMask &pm, float *gk, float *gb, float *ws,
                                 hipStream_t s, ReduceJob *defer);
+// Weight and bias gradients of two 3D layers of a dense block (one output channel each, own
+// dilations) in one pass over x: output channel 0 is the lower layer (gk, group->dil[0]), output
+// channel 1 the upper one (group->gk_up[0], group->dil[1]); g.C is the upper layer's channel
+// count, group->lowest_channels the lower one's; gy holds the two (masked) output gradients as
+// consecutive channels, gb two consecutive bias gradients.  No grad_input is touched.
+bool fast_backward_k_pair_supported_3d(const Geom &g, const View<const float> &gy, const View<const float> &x);
+hipError_t fast_backward_k_pair_3d(const Geom &g, const View<const float> &gy, const View<const float> &x, float *gk,
+                                   float *gb, float *ws, hipStream_t s, ReduceJob *defer, const LayerGroup *group);
 // the instances for rows longer than a workgroup covers (2D) and for stacks whose offsets do
 // not fit 32 bits; chosen by fast_backward_xkb_2d / _3d, not called directly
 hipError_t fast_backward_xkb_2d_long(const Geom &g, const View<const float> &gy, const View<const float> &x,

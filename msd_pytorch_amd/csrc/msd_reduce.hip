@@ -37,8 +37,9 @@ __global__ __launch_bounds__(256) void reduce_columns_batched(ReduceBatch b)
         const int64_t nk = b.job[j].nk;
         if (col < nk) {
             const int64_t split = b.job[j].split;
-            if (col < split)
-                b.job[j].gk[col] += s;
+            if (col < split) {
+                if (col < b.job[j].valid0) b.job[j].gk[col] += s;
+            }
             else if (col < 2 * split)
                 b.job[j].gk_up[0][col - split] += s;
             else
@@ -65,7 +66,7 @@ hipError_t reduce_columns_batch(const ReduceJob *jobs, int n, hipStream_t s)
         b.first[i] = total;
         total += jobs[i].ncols;
     }
-    for (int i = n; i < kReduceBatch; i++) b.job[i] = ReduceJob{nullptr, nullptr, nullptr, 0, 0, 0, {nullptr, nullptr}, 0};
+    for (int i = n; i < kReduceBatch; i++) b.job[i] = ReduceJob{nullptr, nullptr, nullptr, 0, 0, 0, {nullptr, nullptr}, 0, 0};
     for (int i = n; i <= kReduceBatch; i++) b.first[i] = total;
     b.n = n;
     if (total == 0) return hipSuccess;

@@ -240,6 +240,119 @@ __device__ __forceinline__ void stage_source_rows(const Geom &g, const RowTeams 
     __syncthreads();
 }
 
+// stage_source_rows (no ReLU mask) in two steps, so that a kernel can ask for the next tile's
+// rows while it still works on the current tile: request_source_rows only issues the loads of
+// the first source row of every (co, p, q) (clamped, always valid addresses; nothing else is
+// done with the values), finish_source_rows applies the masks, adds the second and further
+// source rows of the rows that fold, stages the sums and ends with a workgroup barrier.
+template <int NDIM, int WOUT, int V>
+__device__ __forceinline__ void request_source_rows(const Geom &g, const View<const float> &gy, int b, int z, int y,
+                                                    int lane, float (&m)[WOUT][RowTaps<NDIM>::NPQ][V],
+                                                    const UpperDilations up = UpperDilations{{0, 0}})
+{
+    constexpr int NZ = Taps<NDIM>::NZ;
+    const int x0 = min(lane * V, g.W - V);
+#pragma unroll
+    for (int co = 0; co < WOUT; co++) {
+        const int dil = dilation_of(g, up, co);
+        const AxisSources sz = NDIM == 3 ? adjoint_sources(z, g.D, dil) : single_source();
+        const AxisSources sy = adjoint_sources(y, g.H, dil);
+        const float *gc = gy.p + (int64_t)b * gy.sb + (int64_t)co * gy.sc + x0;
+#pragma unroll
+        for (int p = 0; p < NZ; p++)
+#pragma unroll
+            for (int q = 0; q < 3; q++) {
+                const int cz = min(max(sz.c[p][0], 0), g.D - 1), cy = min(max(sy.c[q][0], 0), g.H - 1);
+                load_vec<V>(gc + (int64_t)cz * gy.sz + (int64_t)cy * gy.sy, m[co][p * 3 + q]);
+            }
+    }
+}
+
+template <int NDIM, int WOUT, int V>
+__device__ __forceinline__ void finish_source_rows(const Geom &g, const RowTeams &rt, const View<const float> &gy, int b,
+                                                   int z, int y, int lane, bool act, float *__restrict__ S,
+                                                   const float (&m)[WOUT][RowTaps<NDIM>::NPQ][V],
+                                                   float (&own)[WOUT][RowTaps<NDIM>::NPQ][V],
+                                                   const UpperDilations up = UpperDilations{{0, 0}})
+{
+    constexpr int NZ = Taps<NDIM>::NZ, NPQ = RowTaps<NDIM>::NPQ;
+    const int x0 = min(lane * V, g.W - V);
+    float s[WOUT][NPQ][V];
+    bool any_folds = false;
+#pragma unroll
+    for (int co = 0; co < WOUT; co++) {
+        const int dil = dilation_of(g, up, co);
+        const AxisSources sz = NDIM == 3 ? adjoint_sources(z, g.D, dil) : single_source();
+        const AxisSources sy = adjoint_sources(y, g.H, dil);
+        any_folds = any_folds || y < dil || y + dil >= g.H || (NDIM == 3 && (z < dil || z + dil >= g.D));
+#pragma unroll
+        for (int p = 0; p < NZ; p++)
+#pragma unroll
+            for (int q = 0; q < 3; q++)
+#pragma unroll
+                for (int i = 0; i < V; i++)
+                    s[co][p * 3 + q][i] = sz.ok[p][0] && sy.ok[q][0] && act ? m[co][p * 3 + q][i] : 0.f;
+    }
+    if (any_folds) {
+        // rows within dil of a y (or z) border: the other source rows of every output channel,
+        // all requested before the first is used
+        float e[WOUT][NPQ][NDIM == 3 ? 3 : 1][V];
+#pragma unroll
+        for (int co = 0; co < WOUT; co++) {
+            const int dil = dilation_of(g, up, co);
+            const AxisSources sz = NDIM == 3 ? adjoint_sources(z, g.D, dil) : single_source();
+            const AxisSources sy = adjoint_sources(y, g.H, dil);
+            const float *gc = gy.p + (int64_t)b * gy.sb + (int64_t)co * gy.sc + x0;
+            auto row = [&](int cz, int cy, float (&d)[V]) {
+                cz = min(max(cz, 0), g.D - 1);
+                cy = min(max(cy, 0), g.H - 1);
+                load_vec<V>(gc + (int64_t)cz * gy.sz + (int64_t)cy * gy.sy, d);
+            };
+#pragma unroll
+            for (int p = 0; p < NZ; p++)
+#pragma unroll
+                for (int q = 0; q < 3; q++) {
+                    row(sz.c[p][0], sy.c[q][1], e[co][p * 3 + q][0]);
+                    if (NDIM == 3) {
+                        row(sz.c[p][1], sy.c[q][0], e[co][p * 3 + q][1]);
+                        row(sz.c[p][1], sy.c[q][1], e[co][p * 3 + q][2]);
+                    }
+                }
+        }
+#pragma unroll
+        for (int co = 0; co < WOUT; co++) {
+            const int dil = dilation_of(g, up, co);
+            const AxisSources sz = NDIM == 3 ? adjoint_sources(z, g.D, dil) : single_source();
+            const AxisSources sy = adjoint_sources(y, g.H, dil);
+#pragma unroll
+            for (int p = 0; p < NZ; p++)
+#pragma unroll
+                for (int q = 0; q < 3; q++)
+#pragma unroll
+                    for (int i = 0; i < V; i++) {
+                        // (the same order of additions as stage_source_rows)
+                        s[co][p * 3 + q][i] += sz.ok[p][0] && sy.ok[q][1] && act ? e[co][p * 3 + q][0][i] : 0.f;
+                        if (NDIM == 3) {
+                            s[co][p * 3 + q][i] += sz.ok[p][1] && sy.ok[q][0] && act ? e[co][p * 3 + q][1][i] : 0.f;
+                            s[co][p * 3 + q][i] += sz.ok[p][1] && sy.ok[q][1] && act ? e[co][p * 3 + q][2][i] : 0.f;
+                        }
+                    }
+        }
+    }
+#pragma unroll
+    for (int co = 0; co < WOUT; co++)
+#pragma unroll
+        for (int pq = 0; pq < NPQ; pq++) {
+            float *row = S + (size_t)(co * NPQ + pq) * V * rt.lpr;
+#pragma unroll
+            for (int i = 0; i < V; i++) {
+                own[co][pq][i] = s[co][pq][i];
+                row[i * rt.lpr + lane] = s[co][pq][i];
+            }
+        }
+    __syncthreads();
+}
+
 // Segment variant of stage_source_rows (no ReLU mask): the team owns voxels
 // [xs, xs + V * lpr) of row (z, y).  A staged row holds the segment in the usual layout, then
 // `dil` values to the left of it and `dil` values to the right (zeros outside the row), which

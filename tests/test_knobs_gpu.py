@@ -274,3 +274,46 @@ def test_paired_and_single_backward_agree_when_the_input_needs_no_gradient():
             grads[pair] = [bd.grad.clone()] + [w.grad.clone() for w in wd]
     for a, b, c in zip(grads[0], grads[1], grads[3]):
         assert rel_err(a, b) <= 1e-5 and rel_err(a, c) <= 1e-5
+
+
+# 3D blocks of one-channel layers: the reverse loop as a chain of backward_x launches with the
+# weight gradients two layers per pass beside it ("block.split3d": on a second stream, on the
+# caller's stream, or off = one fused launch per layer).  (size, c_in, depth, batch, dilations)
+SPLIT_BLOCKS_3D = [
+    ((6, 7, 64), 1, 6, 1, [1, 2, 3]),            # even depth: pairs down to layers (1, 0)
+    ((5, 9, 128), 2, 7, 2, [3, 1, 2, 5]),        # odd depth: the lowest layer on its own; batch of 2
+    ((12, 10, 128), 1, 9, 1, [10, 1, 7, 2]),     # dilations up to the extents: every row folds
+    ((4, 6, 256), 3, 4, 1, [2, 1]),              # rows of 256 voxels: one row per workgroup
+    ((9, 8, 64), 15, 5, 1, [1, 4, 2]),           # 16 to 20 channels: two blocks of 16 in the upper pairs
+    ((6, 6, 64), 62, 5, 1, [2, 3]),              # 63 to 67 channels: two chunks of the grid
+    ((7, 5, 96), 1, 5, 1, [1, 2]),               # rows the row kernels take with half-empty waves
+]
+SPLIT_MODES = {"two-streams": {"block.split3d": 1}, "one-stream": {"block.split3d": 2}, "fused": {"block.split3d": 0},
+               "default": {}}
+
+
+@pytest.mark.parametrize("mode", list(SPLIT_MODES))
+@pytest.mark.parametrize("case", SPLIT_BLOCKS_3D, ids=lambda c: "x".join(map(str, c[0])) + "-c%d-d%d" % (c[1], c[2]))
+def test_block_backward_3d_chain_and_paired_weight_gradients(case, mode):
+    size, c_in, depth, batch, dilations = case
+    dilations = [dilations[i % len(dilations)] for i in range(depth)]
+    with tuning(SPLIT_MODES[mode]):
+        check_block(3, size, c_in, 1, depth, batch, dilations=dilations, seed=17)
+
+
+def test_block_backward_3d_modes_give_the_same_bits_run_after_run():
+    # the second stream changes when things run, not what is added in which order
+    from msd_pytorch_amd.msd_block import msd_block
+    from parity import block_problem
+    x, dil, bias, ws, g = block_problem(3, (10, 12, 128), 1, 1, 8, 1, seed=23)
+    runs = []
+    for mode in ("two-streams", "two-streams", "one-stream"):
+        with tuning(SPLIT_MODES[mode]):
+            xd = x.cuda().requires_grad_(True)
+            bd = bias.cuda().requires_grad_(True)
+            wd = [w.cuda().requires_grad_(True) for w in ws]
+            msd_block(xd, dil, bd, *wd).backward(g.cuda())
+            torch.cuda.synchronize()
+            runs.append([xd.grad.clone(), bd.grad.clone()] + [w.grad.clone() for w in wd])
+    for other in runs[1:]:
+        assert all(torch.equal(a, b) for a, b in zip(runs[0], other))
