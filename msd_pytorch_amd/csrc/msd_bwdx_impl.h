@@ -8,16 +8,18 @@
 // loads overlap.  Algorithmic traffic: (2C + 2w) * N * 4 bytes.
 #pragma once
 #include "msd_kernels.h"
+
+#include <algorithm>
 #include "msd_rows.h"
 
 namespace msd {
 
 namespace bwdx {
 
-template <int NDIM, bool RELU, int WOUT, int V, int U, int MAXT>
-__global__ __launch_bounds__(MAXT) void bwdx_rows(Geom g, RowTeams rt, int cch, int remap, View<const float> out,
-                                                  View<const float> gy, const float *__restrict__ k, View<float> gx,
-                                                  PostMask pm)
+template <int NDIM, bool RELU, int WOUT, int V, int U>
+__device__ __forceinline__ void bwdx_rows_body(const Geom &g, const RowTeams &rt, int cch, int remap,
+                                               const View<const float> &out, const View<const float> &gy,
+                                               const float *__restrict__ k, const View<float> &gx, const PostMask &pm)
 {
     extern __shared__ float lds[];
     constexpr int K = Taps<NDIM>::K, NPQ = RowTaps<NDIM>::NPQ;
@@ -97,6 +99,14 @@ __global__ __launch_bounds__(MAXT) void bwdx_rows(Geom g, RowTeams rt, int cch, 
 }
 
 constexpr size_t kMaxLds = 64 * 1024;
+
+template <int NDIM, bool RELU, int WOUT, int V, int U, int MAXT>
+__global__ __launch_bounds__(MAXT) void bwdx_rows(Geom g, RowTeams rt, int cch, int remap, View<const float> out,
+                                                  View<const float> gy, const float *__restrict__ k, View<float> gx,
+                                                  PostMask pm)
+{
+    bwdx_rows_body<NDIM, RELU, WOUT, V, U>(g, rt, cch, remap, out, gy, k, gx, pm);
+}
 
 template <int NDIM, bool RELU, int WOUT, int V, int U>
 hipError_t launch(const Geom &g, const View<const float> &out, const View<const float> &gy, const float *k,
