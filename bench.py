@@ -133,7 +133,7 @@ def make_model(name, torch):
     return model
 
 
-def algorithmic_work(name, fused, paired=False, triple_from=32, kpairs=False):
+def algorithmic_work(name, fused, paired=False, triple_from=32, kpairs=False, chainpairs=False):
     """Per-step algorithmic bytes and flops of each kernel class, fp32, per layer with C input
     and w output channels over N voxels and K = 9 or 27 taps:
     bytes: forward (C + w) N 4, backward_x (2C + 2w) N 4, backward_k+bias (C + 2w) N 4, the fused
@@ -153,6 +153,10 @@ def algorithmic_work(name, fused, paired=False, triple_from=32, kpairs=False):
     weight and bias gradients of two layers per pass over x beside it (layers depth-1 and depth-2,
     ... down to 1 and 0; an odd lowest layer alone): a pair reads the C input channels of its
     upper layer once and two output gradients, (C + 4) N 4 bytes.
+    `chainpairs`: that chain takes the same pairs: the upper layer over the one channel the lower
+    layer wrote, 4 N 4 bytes (the channel's gradient read and written, its activation, the upper
+    output gradient), then one read-modify-write pass over the C - 1 channels below with both
+    layers' shares, (2 (C - 1) + 2) N 4 bytes.
     Returns (bytes per class, flops per class, voxels per step)."""
     kind, ndim, c_in, c_out, depth, width, batch, spatial, adam = WORKLOADS[name]
     n = batch
@@ -187,7 +191,12 @@ def algorithmic_work(name, fused, paired=False, triple_from=32, kpairs=False):
                 nbytes["backward_xkb"] += per_layer
             flops["backward_xkb"] += 2 * op
             continue
-        if i > 0:
+        upper, lower = (depth - 1 - i) % 2 == 0 and i > 0, (depth - 1 - i) % 2 == 1
+        if chainpairs and (upper or lower):
+            if i > 0:                         # (layer 0's pass would only serve a gradient of the block's input)
+                nbytes["backward_x"] += 4 * n * 4 + K * 4 if upper else (2 * C + 2) * n * 4 + 2 * wts
+                flops["backward_x"] += op if i > 1 else 2 * K * n
+        elif i > 0:
             nbytes["backward_x"] += (2 * C + 2 * width) * n * 4 + wts
             flops["backward_x"] += op
         flops["backward_kb"] += op
@@ -331,7 +340,8 @@ def measure(name, args, lib, torch, steps=None, warmup=None, cpu=True):
         split3d = ndim == 3 and width == 1 and totals["backward_xkb"][1] == 0 and \
             0 < totals["backward_kb"][1] // args.steps < depth
         bytes_per_step, flops_per_step, _ = algorithmic_work(name, totals["backward_xkb"][1] > 0, paired, triple_from,
-                                                             kpairs=split3d)
+                                                             kpairs=split3d,
+                                                             chainpairs=split3d and tuned.get("block.chainpair") != "0")
         kernels = {}
         for cls, (ms, launches) in totals.items():
             if launches == 0:
@@ -357,8 +367,8 @@ def measure(name, args, lib, torch, steps=None, warmup=None, cpu=True):
         # the committed counter figures describe the library's default launch shapes
         traffic, source = ({}, None) if args.tune else profiled_traffic(name, split3d)
         if split3d:
-            result["config"]["backward"] = ("chain of backward_x launches; weight gradients two layers per pass on a "
-                                            "second stream (kernel classes timed on one stream)")
+            result["config"]["backward"] = ("chain of backward_x launches (two layers per pass); weight gradients two "
+                                            "layers per pass on a second stream (kernel classes timed on one stream)")
         per_launch, profiled_calls = traffic.get(dominant, (None, None))
         stale = per_launch is not None and profiled_calls is not None and profiled_calls != dom["calls_per_step"]
         if stale:

@@ -17,9 +17,9 @@ const char *const kKnobNames[kKnobCount] = {
     "xcd_remap", "bwdk.vec2d", "bwdk.vec3d", "bwdk.blocks",
     "fwd.vec2d", "fwd.vec3d", "fwd.split", "fwd.rows2d", "bwdk.rows", "block.fuse",
     "block.defer", "bwdk.interleave", "block.snake", "fwd.class3d", "fwd.lattice3d",
-    "block.pair", "block.triple", "final.tiled", "block.split3d",
+    "block.pair", "block.triple", "final.tiled", "block.split3d", "block.chainpair",
 };
-static_assert(kKnobBlockSplit3d + 1 == kKnobCount, "one name per knob, in the order of the enum");
+static_assert(kKnobBlockChainPair + 1 == kKnobCount, "one name per knob, in the order of the enum");
 int g_knobs[kKnobCount];
 // every knob starts at "library default"
 const bool g_knobs_ready = [] {
@@ -1030,14 +1030,55 @@ int block_backward_split3d(const char *fn, const BlockArgs &a, int64_t c_in, con
         msd::LayerGroup group;
         msd::View<const float> gy;
     };
+    // The chain takes the same pairs where it can: the upper layer first finishes the one channel
+    // the lower layer wrote (a launch over that channel alone), then one read-modify-write pass
+    // over the channels below adds both layers' shares (grad_input is read and written once per
+    // two layers).  (128^3, depth 50: the chain's launches take 3.2 instead of 4.7 ms.)
+    struct Step {
+        msd::Geom g;                              // the upper layer over the lower one's channel / the pair's pass
+        msd::LayerGroup group;
+        msd::View<float> gx;
+        const float *k;
+        msd::PostMask pm;
+    };
     std::vector<Pair> pairs(a.depth);             // pairs[l]: layers (l + 1, l), l the lower one
+    std::vector<Step> steps(a.depth);             // [upper]: its one channel; [lower]: the pair's pass
     std::vector<msd::Geom> chain(a.depth);
+    bool chain_pairs = msd::knob(msd::kKnobBlockChainPair, 1) != 0 && x.sx == 1;
+    const int64_t taps = 27;
     for (int i = a.depth - 1; i >= 0; i--) {
         const int64_t first = c_in + i;           // channels layer i reads; its output is channel `first`
         MSD_TRY(make_geom(fn, a.dtype, a.ndim, a.batch, first, 1, a.spatial, (int)a.dilations[i], true, &chain[i]));
         const msd::View<const float> gy{gx.p + first * gx.sc, gx.sb, gx.sc, gx.sz, gx.sy, gx.sx};
         if ((i > 0 || need_input_grad) && !msd::fast_backward_x_supported(chain[i], false, gy, gy, gx)) return MSD_OK;
         const bool lower = (a.depth - 1 - i) % 2 == 1;
+        if (!lower && i > 0) {
+            // layer i over channel first - 1 alone, masked by the activation that channel holds
+            Step &st = steps[i];
+            MSD_TRY(make_geom(fn, a.dtype, a.ndim, a.batch, 1, 1, a.spatial, (int)a.dilations[i], true, &st.g));
+            st.gx = msd::View<float>{gx.p + (first - 1) * gx.sc, gx.sb, gx.sc, gx.sz, gx.sy, gx.sx};
+            st.k = (const float *)weights[i] + (first - 1) * taps;
+            st.pm = msd::PostMask{0, {x.p + (first - 1) * x.sc, x.sb, x.sc, x.sz, x.sy, x.sx}};
+            chain_pairs = chain_pairs && msd::fast_backward_x_supported(st.g, false, gy, gy, st.gx);
+        }
+        if (lower) {
+            Step &st = steps[i];
+            const int du = (int)a.dilations[i + 1], dl = (int)a.dilations[i];
+            MSD_TRY(make_geom(fn, a.dtype, a.ndim, a.batch, first, 2, a.spatial, dl, true, &st.g));
+            st.group.n = 2;
+            st.group.dil[0] = dl;
+            st.group.dil[1] = du;
+            st.group.dil[2] = 0;
+            st.group.k_up[0] = (const float *)weights[i + 1];
+            st.group.k_up[1] = nullptr;
+            st.group.gk_up[0] = st.group.gk_up[1] = nullptr;
+            st.group.lowest_channels = 0;
+            st.gx = gx;
+            st.k = (const float *)weights[i];
+            st.pm = i > 0 ? msd::PostMask{(int)(first - 1), x} : msd::PostMask{(int)first, {nullptr, 0, 0, 0, 0, 0}};
+            if (i > 0 || need_input_grad)
+                chain_pairs = chain_pairs && msd::fast_backward_x_pair_supported_3d(st.g, gy, gx);
+        }
         if (lower) {
             Pair &p = pairs[i];
             const int du = (int)a.dilations[i + 1], dl = (int)a.dilations[i];
@@ -1098,11 +1139,27 @@ int block_backward_split3d(const char *fn, const BlockArgs &a, int64_t c_in, con
                                 (int)a.dilations[i], nullptr, nullptr, gout_i, grads_strides, stack, stack_strides,
                                 grad_weights[i], (char *)grad_bias + i * a.elem, workspace, workspace_bytes, ks));
         }
-        if (i > 0 || need_input_grad)
+        const msd::View<const float> gy{gx.p + first * gx.sc, gx.sb, gx.sc, gx.sz, gx.sy, gx.sx};
+        if (chain_pairs && !lower && i > 0) {
+            const Step &st = steps[i];
+            ProfileScope scope(1, main);
+            const hipError_t e = msd::fast_backward_x_3d(st.g, false, gy, gy, st.k, st.gx, st.pm, main);
+            if (e != hipSuccess) return hip_fail(fn, e);
+            masked = true;
+        } else if (chain_pairs && lower) {
+            if (i > 0 || need_input_grad) {
+                const Step &st = steps[i];
+                ProfileScope scope(1, main);
+                const hipError_t e = msd::fast_backward_x_pair_3d(st.g, gy, st.k, st.gx, st.pm, main, &st.group);
+                if (e != hipSuccess) return hip_fail(fn, e);
+                masked = i > 0;
+            }
+        } else if (i > 0 || need_input_grad) {
             MSD_TRY(backward_x("conv_backward_x", false, a.dtype, a.ndim, a.batch, first, 1, a.spatial,
                                (int)a.dilations[i], nullptr, nullptr, gout_i, grads_strides, weights[i], grads,
                                grads_strides, main, i > 0 ? (int)(first - 1) : (int)first, i > 0 ? stack : nullptr,
                                stack_strides, &masked));
+        }
     }
     MSD_TRY(pending->flush(fn));
     if (side) {

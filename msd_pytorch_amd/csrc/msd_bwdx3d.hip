@@ -15,4 +15,15 @@ hipError_t fast_backward_x_3d(const Geom &g, bool relu, const View<const float> 
     return bwdx::fast_backward_x_nd<3>(g, relu, out, gy, k, gx, pm, s);
 }
 
+bool fast_backward_x_pair_supported_3d(const Geom &g, const View<const float> &gy, const View<float> &gx)
+{
+    return bwdx::pair_vec<3>(g, gy, gx) != 0;
+}
+
+hipError_t fast_backward_x_pair_3d(const Geom &g, const View<const float> &gy, const float *k, const View<float> &gx,
+                                   const PostMask &pm, hipStream_t s, const LayerGroup *group)
+{
+    return bwdx::pair_nd<3>(g, gy, k, gx, pm, s, group);
+}
+
 }  // namespace msd

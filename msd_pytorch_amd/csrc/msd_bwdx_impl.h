@@ -98,6 +98,136 @@ __device__ __forceinline__ void bwdx_rows_body(const Geom &g, const RowTeams &rt
     }
 }
 
+// Two layers of a dense block per pass (WOUT == 2: channel 0 with the Geom's dilation and the
+// weights k, channel 1 with up.d[0] and k1, both [C][K] arrays over the channels the layers
+// share), with the channel loop as a software pipeline: 108 multiply-adds per voxel and channel
+// leave the memory latency to be hidden by the wave itself, so the loads run kAhead steps of U
+// channels ahead of the arithmetic in a ring of register sets (V floats per channel: the ring
+// is small next to the gathered taps).  A set is loaded into again two steps after its
+// channels were stored: overwriting the registers of stores that were only just issued would
+// have to wait for them.  Nothing in the loop is under a condition: the last step repeats the
+// last channel where the count is not a multiple of U (same values in, same values out), and
+// the ReLU mask of the layer below comes from one load before the loop; the number of accesses
+// in flight is then the same on every path and the waits are for exactly the set that is needed.
+constexpr int kRingSets = 5;                     // kAhead = kRingSets - 2 steps
+
+template <int NDIM, int V, int U>
+__device__ __forceinline__ void bwdx_pair_body(const Geom &g, const RowTeams &rt, int cch, int remap,
+                                               const View<const float> &gy, const float *__restrict__ k,
+                                               const float *__restrict__ k1, const UpperDilations &up,
+                                               const View<float> &gx, const PostMask &pm)
+{
+    extern __shared__ float lds[];
+    constexpr int WOUT = 2, K = Taps<NDIM>::K, NPQ = RowTaps<NDIM>::NPQ, NS = kRingSets;
+    const int team = threadIdx.x / rt.lpr, lane = threadIdx.x % rt.lpr;
+    const int lb = block_for_xcd(blockIdx.x, gridDim.x, remap);
+    if (lb * rt.rpw >= rt.nrows) return;   // padding block (whole workgroup)
+    const int row = lb * rt.rpw + team;
+    const int x0 = lane * V;
+    const bool act = row < rt.nrows && x0 < g.W;
+    const int rr = min(row, rt.nrows - 1);
+    const int y = rr % g.H, z = rr / g.H;
+    const int b = blockIdx.y;
+    const int c0 = blockIdx.z * cch;
+    const int c1 = min(c0 + cch, g.C);
+
+    float A[WOUT][K][V];
+    {
+        float *S = lds + (size_t)team * WOUT * NPQ * V * rt.lpr;
+        float own[WOUT][NPQ][V];
+        stage_source_rows<NDIM, false, WOUT, V>(g, rt, gy, gy, b, z, y, lane, act, S, own, up);
+#pragma unroll
+        for (int i = 0; i < V; i++) {
+#pragma unroll
+            for (int co = 0; co < WOUT; co++) {
+                const SideTaps<V> side(x0 + i, g.W, dilation_of(g, up, co), rt.lpr);
+#pragma unroll
+                for (int pq = 0; pq < NPQ; pq++) {
+                    side.read(S + (size_t)(co * NPQ + pq) * V * rt.lpr, A[co][pq * 3 + 0][i], A[co][pq * 3 + 2][i]);
+                    A[co][pq * 3 + 1][i] = own[co][pq][i];
+                }
+            }
+        }
+    }
+    if (!act) return;
+
+    const int64_t spatial = (int64_t)b * gx.sb + (int64_t)z * gx.sz + (int64_t)y * gx.sy + x0;
+    float *gp = gx.p + spatial;
+    // channels from pm.from on are outputs of the layer below: their gradient is complete with
+    // this update, so its ReLU mask is applied on the way out.  (The dense block masks the one
+    // channel that ends the pass; `keep` is that channel's mask.)
+    bool keep[V];
+    {
+        float a[V];
+        load_vec<V>(pm.from < c1 ? pm.act.p + (int64_t)b * pm.act.sb + (int64_t)(c1 - 1) * pm.act.sc +
+                                       (int64_t)z * pm.act.sz + (int64_t)y * pm.act.sy + x0
+                                 : gp,
+                    a);
+#pragma unroll
+        for (int i = 0; i < V; i++) keep[i] = !(pm.from < c1) || 0.f < a[i];
+    }
+
+    float ring[NS][U][V];
+    auto load_set = [&](int set, int ci) {
+#pragma unroll
+        for (int u = 0; u < U; u++) load_vec<V>(gp + (int64_t)min(ci + u, c1 - 1) * gx.sc, ring[set][u]);
+    };
+    // The weights are wave-uniform: scalar loads into scalar registers, which complete in any
+    // order, so a wait for some of them is a wait for all.  They are therefore asked for one
+    // stage (one layer's 27 taps of one channel) ahead, into the registers of the other layer:
+    // the wait before a stage's arithmetic finds its weights long since there and only has the
+    // next stage's to sit out, behind 27 multiply-adds per voxel.
+    typedef const __attribute__((address_space(4))) float *const_floats_t;
+    const const_floats_t kw0 = (const_floats_t)(uintptr_t)k, kw1 = (const_floats_t)(uintptr_t)k1;
+    float w0[K], w1[K];
+    auto request = [&](const_floats_t kw, int ch, float (&w)[K]) {
+#pragma unroll
+        for (int t = 0; t < K; t++) w[t] = kw[(int64_t)ch * K + t];
+    };
+    auto finish_set = [&](int set, int ci) {
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int cu = min(ci + u, c1 - 1), cn = min(ci + u + 1, c1 - 1);
+            float s[V];
+#pragma unroll
+            for (int i = 0; i < V; i++) s[i] = 0.f;
+            request(kw1, cu, w1);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int t = 0; t < K; t++)
+#pragma unroll
+                for (int i = 0; i < V; i++) s[i] += w0[t] * A[0][t][i];
+            __builtin_amdgcn_sched_barrier(0);
+            request(kw0, cn, w0);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int t = 0; t < K; t++)
+#pragma unroll
+                for (int i = 0; i < V; i++) s[i] += w1[t] * A[1][t][i];
+            const bool last = cu == c1 - 1;
+#pragma unroll
+            for (int i = 0; i < V; i++) {
+                ring[set][u][i] += s[i];
+                ring[set][u][i] = last && !keep[i] ? 0.f : ring[set][u][i];
+            }
+            store_vec<V>(gp + (int64_t)cu * gx.sc, ring[set][u]);
+        }
+    };
+    request(kw0, c0, w0);
+#pragma unroll
+    for (int j = 0; j < NS - 2; j++) load_set(j, c0 + j * U);
+    for (int ci = c0;;) {
+#pragma unroll
+        for (int j = 0; j < NS; j++) {
+            load_set((j + NS - 2) % NS, ci + (NS - 2) * U);
+            __builtin_amdgcn_sched_barrier(0);   // (the loads stay ahead of the arithmetic)
+            finish_set(j, ci);
+            ci += U;
+            if (ci >= c1) return;
+        }
+    }
+}
+
 constexpr size_t kMaxLds = 64 * 1024;
 
 template <int NDIM, bool RELU, int WOUT, int V, int U, int MAXT>
@@ -108,9 +238,18 @@ __global__ __launch_bounds__(MAXT) void bwdx_rows(Geom g, RowTeams rt, int cch, 
     bwdx_rows_body<NDIM, RELU, WOUT, V, U>(g, rt, cch, remap, out, gy, k, gx, pm);
 }
 
-template <int NDIM, bool RELU, int WOUT, int V, int U>
+template <int NDIM, int V, int U>
+__global__ __launch_bounds__(256) void bwdx_rows_pair(Geom g, RowTeams rt, int cch, int remap, View<const float> gy,
+                                                      const float *__restrict__ k, const float *__restrict__ k1,
+                                                      UpperDilations up, View<float> gx, PostMask pm)
+{
+    bwdx_pair_body<NDIM, V, U>(g, rt, cch, remap, gy, k, k1, up, gx, pm);
+}
+
+template <int NDIM, bool RELU, int WOUT, int V, int U, bool PAIR = false>
 hipError_t launch(const Geom &g, const View<const float> &out, const View<const float> &gy, const float *k,
-                  const View<float> &gx, const PostMask &pm, hipStream_t s)
+                  const View<float> &gx, const PostMask &pm, hipStream_t s, const float *k1 = nullptr,
+                  const UpperDilations up = UpperDilations{{0, 0}})
 {
     RowTeams rt;
     make_row_teams(g, V, &rt);
@@ -125,6 +264,12 @@ hipError_t launch(const Geom &g, const View<const float> &out, const View<const 
     chunks = (g.C + cch - 1) / cch;
     const int remap = knob(kKnobXcdRemap, 1);
     const dim3 grid(remap ? xcd_grid(nb) : nb, g.B, chunks);
+    if constexpr (PAIR) {
+        if (rt.lpr * rt.rpw > 256) return hipErrorInvalidConfiguration;   // excluded by pair_supported()
+        hipLaunchKernelGGL((bwdx_rows_pair<NDIM, V, U>), grid, dim3(rt.lpr * rt.rpw), lds, s, g, rt, cch, remap, gy, k,
+                           k1, up, gx, pm);
+        return hipGetLastError();
+    }
     if (rt.lpr * rt.rpw <= 256) {
         hipLaunchKernelGGL((bwdx_rows<NDIM, RELU, WOUT, V, U, 256>), grid, dim3(rt.lpr * rt.rpw), lds,
                            s, g, rt, cch, remap, out, gy, k, gx, pm);
@@ -201,6 +346,50 @@ bool fast_backward_x_supported_nd(const Geom &g, bool relu, const View<const flo
     if (g.Wd > 2) return false;
     if (gx.sx != 1 || gy.sx != 1 || (relu && out.sx != 1)) return false;
     return choose_vec<NDIM>(g, relu, g.Wd, 4, out, gy, gx) != 0;
+}
+
+// Two layers of a dense block (one output channel each) over the g.C input channels they
+// share: g.dil and k are the lower layer's, group->dil[1] and group->k_up[0] the upper one's;
+// gy holds the two masked output gradients as consecutive channels (lower first).
+template <int NDIM>
+int pair_vec(const Geom &g, const View<const float> &gy, const View<float> &gx)
+{
+    if (g.Wd != 2 || gx.sx != 1 || gy.sx != 1) return 0;
+    const int vmax = knob(NDIM == 3 ? kKnobBwdxVec3d : kKnobBwdxVec2d, NDIM == 3 ? 1 : 4);
+    for (int pass = 0; pass < 2; pass++)
+        for (int v = 4; v >= 1; v /= 2) {
+            if (pass == 0 && v > vmax) continue;
+            if (!rows_aligned(gx, g.W, v) || !rows_aligned(gy, g.W, v) || !fits<NDIM>(g, v, 2)) continue;
+            RowTeams rt;
+            make_row_teams(g, v, &rt);
+            if (rt.lpr * rt.rpw <= 256) return v;
+        }
+    return 0;
+}
+
+template <int NDIM, int V>
+hipError_t pair_unroll(const Geom &g, const View<const float> &gy, const float *k, const View<float> &gx,
+                       const PostMask &pm, hipStream_t s, const float *k1, const UpperDilations up)
+{
+    const int u = knob(NDIM == 3 ? kKnobBwdxUnroll3d : kKnobBwdxUnroll2d, 2);
+    if (u <= 2) return launch<NDIM, false, 2, V, 2, true>(g, gy, gy, k, gx, pm, s, k1, up);
+    return launch<NDIM, false, 2, V, 4, true>(g, gy, gy, k, gx, pm, s, k1, up);
+}
+
+template <int NDIM>
+hipError_t pair_nd(const Geom &g, const View<const float> &gy, const float *k, const View<float> &gx, const PostMask &pm,
+                   hipStream_t s, const LayerGroup *group)
+{
+    if (!group || group->n != 2 || !group->k_up[0]) return hipErrorInvalidValue;
+    if (pm.from < g.C - 1) return hipErrorInvalidValue;   // (at most the channel that ends the pass is masked)
+    Geom g2 = g;
+    g2.dil = group->dil[0];
+    const UpperDilations up{{group->dil[1], 0}};
+    const int v = pair_vec<NDIM>(g2, gy, gx);
+    if (v == 4) return pair_unroll<NDIM, 4>(g2, gy, k, gx, pm, s, group->k_up[0], up);
+    if (v == 2) return pair_unroll<NDIM, 2>(g2, gy, k, gx, pm, s, group->k_up[0], up);
+    if (v == 1) return pair_unroll<NDIM, 1>(g2, gy, k, gx, pm, s, group->k_up[0], up);
+    return hipErrorInvalidConfiguration;
 }
 
 template <int NDIM>

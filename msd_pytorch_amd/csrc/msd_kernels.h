@@ -61,7 +61,7 @@ enum Knob {
     kKnobXcdRemap, kKnobBwdkVec2d, kKnobBwdkVec3d, kKnobBwdkBlocks,
     kKnobFwdVec2d, kKnobFwdVec3d, kKnobFwdSplit, kKnobFwdRows2d, kKnobBwdkRows, kKnobBlockFuse,
     kKnobBlockDefer, kKnobBwdkInterleave, kKnobBlockSnake, kKnobFwdClass3d, kKnobFwdLattice3d,
-    kKnobBlockPair, kKnobBlockTriple, kKnobFinalTiled, kKnobBlockSplit3d,
+    kKnobBlockPair, kKnobBlockTriple, kKnobFinalTiled, kKnobBlockSplit3d, kKnobBlockChainPair,
     kKnobCount
 };
 int knob(Knob k, int dflt);
@@ -194,6 +194,14 @@ hipError_t fast_backward_xkb_3d(const Geom &g, const View<const float> &gy, cons
 bool fast_backward_k_pair_supported_3d(const Geom &g, const View<const float> &gy, const View<const float> &x);
 hipError_t fast_backward_k_pair_3d(const Geom &g, const View<const float> &gy, const View<const float> &x, float *gk,
                                    float *gb, float *ws, hipStream_t s, ReduceJob *defer, const LayerGroup *group);
+// grad_input of two 3D layers of a dense block (one output channel each, own dilations) in one
+// read-modify-write pass over the g.C input channels they share: output channel 0 is the lower
+// layer (k, group->dil[0]), output channel 1 the upper one (group->k_up[0], group->dil[1]); gy
+// holds the two (masked) output gradients as consecutive channels.  Per channel and voxel the
+// lower layer's taps are summed first, then the upper one's, and the sum is added to grad_input.
+bool fast_backward_x_pair_supported_3d(const Geom &g, const View<const float> &gy, const View<float> &gx);
+hipError_t fast_backward_x_pair_3d(const Geom &g, const View<const float> &gy, const float *k, const View<float> &gx,
+                                   const PostMask &pm, hipStream_t s, const LayerGroup *group);
 // the instances for rows longer than a workgroup covers (2D) and for stacks whose offsets do
 // not fit 32 bits; chosen by fast_backward_xkb_2d / _3d, not called directly
 hipError_t fast_backward_xkb_2d_long(const Geom &g, const View<const float> &gy, const View<const float> &x,

@@ -109,12 +109,13 @@ def block_problem(ndim, size, c_in, width, depth, batch, dilations=None, seed=0)
     return x, dil, bias, ws, g
 
 
-def check_block(ndim, size, c_in, width, depth, batch, dilations=None, seed=0):
+def check_block(ndim, size, c_in, width, depth, batch, dilations=None, seed=0, input_grad=True):
     """msd_block forward + backward (native layer loops) against the fp64 oracle: the whole
-    stack, grad_input, every weight gradient and the bias gradient."""
+    stack, grad_input (unless the input takes no gradient), every weight gradient and the bias
+    gradient."""
     from msd_pytorch_amd.msd_block import msd_block
     x, dil, bias, ws, g = block_problem(ndim, size, c_in, width, depth, batch, dilations, seed)
-    xd = x.cuda().requires_grad_(True)
+    xd = x.cuda().requires_grad_(input_grad)
     bd = bias.cuda().requires_grad_(True)
     wd = [w.cuda().requires_grad_(True) for w in ws]
     got = msd_block(xd, dil, bd, *wd)
@@ -129,7 +130,10 @@ def check_block(ndim, size, c_in, width, depth, batch, dilations=None, seed=0):
     # mask in an upper layer changes every gradient below it by far more than the tolerance.
     want_gx, want_gb, want_gw = oracle.block_backward(got.detach().double().cpu(), g.double(), dil, bias.double(),
                                                       ws64)
-    assert rel_err(xd.grad, want_gx) <= 1e-4, "grad_input"
+    if input_grad:
+        assert rel_err(xd.grad, want_gx) <= 1e-4, "grad_input"
+    else:
+        assert xd.grad is None
     assert rel_err(bd.grad, want_gb) <= 1e-4, "grad_bias"
     worst = max((rel_err(a.grad, b), i) for i, (a, b) in enumerate(zip(wd, want_gw)))
     assert worst[0] <= 1e-4, "grad_weight of layer %d" % worst[1]

@@ -289,7 +289,7 @@ SPLIT_BLOCKS_3D = [
     ((7, 5, 96), 1, 5, 1, [1, 2]),               # rows the row kernels take with half-empty waves
 ]
 SPLIT_MODES = {"two-streams": {"block.split3d": 1}, "one-stream": {"block.split3d": 2}, "fused": {"block.split3d": 0},
-               "default": {}}
+               "default": {}, "chain-of-single-layers": {"block.split3d": 1, "block.chainpair": 0}}
 
 
 @pytest.mark.parametrize("mode", list(SPLIT_MODES))
@@ -299,6 +299,23 @@ def test_block_backward_3d_chain_and_paired_weight_gradients(case, mode):
     dilations = [dilations[i % len(dilations)] for i in range(depth)]
     with tuning(SPLIT_MODES[mode]):
         check_block(3, size, c_in, 1, depth, batch, dilations=dilations, seed=17)
+
+
+# The chain's two-layer pass by voxels per lane and channels in flight (rows of 128 voxels take
+# any of the three widths).
+@pytest.mark.parametrize("unroll", [2, 4])
+@pytest.mark.parametrize("vec", [1, 2, 4])
+def test_block_backward_3d_paired_chain_by_vector_width(vec, unroll):
+    with tuning({"block.split3d": 1, "bwdx.vec3d": vec, "bwdx.unroll3d": unroll}):
+        check_block(3, (6, 5, 128), 2, 1, 7, 1, dilations=[2, 1, 3, 1, 5, 2, 4], seed=29)
+        check_block(3, (4, 9, 128), 1, 1, 4, 2, dilations=[1, 3, 2, 4], seed=31)
+
+
+def test_block_backward_3d_without_input_gradient():
+    # the lowest pair then skips its pass over the block's input channels
+    for depth in (4, 5):
+        with tuning({"block.split3d": 1}):
+            check_block(3, (5, 6, 64), 2, 1, depth, 1, dilations=[1, 2, 3, 1, 2][:depth], seed=37, input_grad=False)
 
 
 def test_block_backward_3d_modes_give_the_same_bits_run_after_run():

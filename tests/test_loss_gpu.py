@@ -61,6 +61,26 @@ def test_fused_loss_matches_torch(batch, c_in, c_out, spatial, kind, dtype):
     check_fused_loss(batch, c_in, c_out, spatial, kind, dtype)
 
 
+# One small case per compiled form of the single-read kernel: voxels per lane (4: plane size a
+# multiple of four and at most 64 channels; 2: even planes otherwise; 1: odd planes) x channels
+# per wave and pass (8 up to 64 channels, 16 above) x output channels (1, 2, 3 or 4) x loss.
+SINGLE_READ_FORMS = [
+    # (c_in, spatial)
+    (20, (8, 16)),      # 4 voxels, 8 channels
+    (20, (6, 7)),       # 2 voxels, 8 channels
+    (20, (5, 7)),       # 1 voxel,  8 channels
+    (70, (6, 8)),       # 2 voxels, 16 channels
+    (70, (5, 7)),       # 1 voxel,  16 channels
+]
+
+
+@pytest.mark.parametrize("kind", ["mse", "l1", "nll"])
+@pytest.mark.parametrize("c_out", [1, 2, 3])
+@pytest.mark.parametrize("c_in,spatial", SINGLE_READ_FORMS)
+def test_fused_loss_every_form_of_the_single_read_kernel(c_in, spatial, c_out, kind):
+    check_fused_loss(2, c_in, c_out, spatial, kind, torch.float32)
+
+
 @pytest.mark.parametrize("kind", ["mse", "l1", "nll"])
 @pytest.mark.parametrize("batch,c_in,c_out,spatial", CASES)
 def test_fused_loss_walking_the_stack_twice_matches_torch(batch, c_in, c_out, spatial, kind):
