@@ -35,6 +35,13 @@ __device__ __forceinline__ void bwdx_rows_body(const Geom &g, const RowTeams &rt
     const int c0 = blockIdx.z * cch;
     const int c1 = min(c0 + cch, g.C);
 
+    // the first channels of grad_input are asked for before the gather: their latency passes
+    // behind the gather's (lanes outside the image ask for a valid address and drop the values)
+    float *gp = gx.p + (int64_t)b * gx.sb + (int64_t)z * gx.sz + (int64_t)y * gx.sy + min(x0, g.W - V);
+    float first[U][V];
+#pragma unroll
+    for (int u = 0; u < U; u++) load_vec<V>(gp + (int64_t)min(c0 + u, c1 - 1) * gx.sc, first[u]);
+
     // adjoint gather, kept in registers for the whole channel loop
     float A[WOUT][K][V];
     {
@@ -55,14 +62,18 @@ __device__ __forceinline__ void bwdx_rows_body(const Geom &g, const RowTeams &rt
     }
     if (!act) return;
 
-    float *gp = gx.p + (int64_t)b * gx.sb + (int64_t)z * gx.sz + (int64_t)y * gx.sy + x0;
     for (int ci = c0; ci < c1; ci += U) {
         float cur[U][V];
         int cu[U];
 #pragma unroll
         for (int u = 0; u < U; u++) {
             cu[u] = min(ci + u, c1 - 1);
-            load_vec<V>(gp + (int64_t)cu[u] * gx.sc, cur[u]);
+            if (ci == c0) {
+#pragma unroll
+                for (int i = 0; i < V; i++) cur[u][i] = first[u][i];
+            } else {
+                load_vec<V>(gp + (int64_t)cu[u] * gx.sc, cur[u]);
+            }
         }
 #pragma unroll
         for (int u = 0; u < U; u++) {
@@ -109,7 +120,13 @@ __device__ __forceinline__ void bwdx_rows_body(const Geom &g, const RowTeams &rt
 // last channel where the count is not a multiple of U (same values in, same values out), and
 // the ReLU mask of the layer below comes from one load before the loop; the number of accesses
 // in flight is then the same on every path and the waits are for exactly the set that is needed.
-constexpr int kRingSets = 5;                     // kAhead = kRingSets - 2 steps
+#ifndef MSD_RING_SETS
+#define MSD_RING_SETS 4
+#endif
+// s_waitcnt for the scalar (and LDS) counter alone: lgkmcnt(0), the vector-memory and export
+// counters at their maxima
+constexpr int kWaitScalarLoads = 0xC07F;
+constexpr int kRingSets = MSD_RING_SETS;                     // kAhead = kRingSets - 2 steps
 
 template <int NDIM, int V, int U>
 __device__ __forceinline__ void bwdx_pair_body(const Geom &g, const RowTeams &rt, int cch, int remap,
@@ -131,6 +148,27 @@ __device__ __forceinline__ void bwdx_pair_body(const Geom &g, const RowTeams &rt
     const int c0 = blockIdx.z * cch;
     const int c1 = min(c0 + cch, g.C);
 
+    // What the channel loop starts with is asked for before the gather, so that its latency
+    // passes behind the gather's (lanes outside the image ask for a valid address and drop the
+    // values): the first steps of the ring, and the activation behind the pass's last channel.
+    // Channels from pm.from on are outputs of the layer below: their gradient is complete with
+    // this update, so its ReLU mask is applied on the way out.  (The dense block masks the one
+    // channel that ends the pass; `keep` is that channel's mask.)
+    const int64_t spatial = (int64_t)b * gx.sb + (int64_t)z * gx.sz + (int64_t)y * gx.sy + min(x0, g.W - V);
+    float *gp = gx.p + spatial;
+    float ring[NS][U][V];
+    auto load_set = [&](int set, int ci) {
+#pragma unroll
+        for (int u = 0; u < U; u++) load_vec<V>(gp + (int64_t)min(ci + u, c1 - 1) * gx.sc, ring[set][u]);
+    };
+#pragma unroll
+    for (int j = 0; j < NS - 2; j++) load_set(j, c0 + j * U);
+    float below[V];
+    load_vec<V>(pm.from < c1 ? pm.act.p + (int64_t)b * pm.act.sb + (int64_t)(c1 - 1) * pm.act.sc +
+                                   (int64_t)z * pm.act.sz + (int64_t)y * pm.act.sy + min(x0, g.W - V)
+                             : gp,
+                below);
+
     float A[WOUT][K][V];
     {
         float *S = lds + (size_t)team * WOUT * NPQ * V * rt.lpr;
@@ -151,27 +189,10 @@ __device__ __forceinline__ void bwdx_pair_body(const Geom &g, const RowTeams &rt
     }
     if (!act) return;
 
-    const int64_t spatial = (int64_t)b * gx.sb + (int64_t)z * gx.sz + (int64_t)y * gx.sy + x0;
-    float *gp = gx.p + spatial;
-    // channels from pm.from on are outputs of the layer below: their gradient is complete with
-    // this update, so its ReLU mask is applied on the way out.  (The dense block masks the one
-    // channel that ends the pass; `keep` is that channel's mask.)
     bool keep[V];
-    {
-        float a[V];
-        load_vec<V>(pm.from < c1 ? pm.act.p + (int64_t)b * pm.act.sb + (int64_t)(c1 - 1) * pm.act.sc +
-                                       (int64_t)z * pm.act.sz + (int64_t)y * pm.act.sy + x0
-                                 : gp,
-                    a);
 #pragma unroll
-        for (int i = 0; i < V; i++) keep[i] = !(pm.from < c1) || 0.f < a[i];
-    }
+    for (int i = 0; i < V; i++) keep[i] = !(pm.from < c1) || 0.f < below[i];
 
-    float ring[NS][U][V];
-    auto load_set = [&](int set, int ci) {
-#pragma unroll
-        for (int u = 0; u < U; u++) load_vec<V>(gp + (int64_t)min(ci + u, c1 - 1) * gx.sc, ring[set][u]);
-    };
     // The weights are wave-uniform: scalar loads into scalar registers, which complete in any
     // order, so a wait for some of them is a wait for all.  They are therefore asked for one
     // stage (one layer's 27 taps of one channel) ahead, into the registers of the other layer:
@@ -191,6 +212,9 @@ __device__ __forceinline__ void bwdx_pair_body(const Geom &g, const RowTeams &rt
             float s[V];
 #pragma unroll
             for (int i = 0; i < V; i++) s[i] = 0.f;
+            // (the explicit wait comes before the next request on purpose: placed by the compiler
+            // it would stand before the first use, behind the request, and wait for that too)
+            __builtin_amdgcn_s_waitcnt(kWaitScalarLoads);
             request(kw1, cu, w1);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -198,6 +222,7 @@ __device__ __forceinline__ void bwdx_pair_body(const Geom &g, const RowTeams &rt
 #pragma unroll
                 for (int i = 0; i < V; i++) s[i] += w0[t] * A[0][t][i];
             __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_waitcnt(kWaitScalarLoads);
             request(kw0, cn, w0);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -214,8 +239,6 @@ __device__ __forceinline__ void bwdx_pair_body(const Geom &g, const RowTeams &rt
         }
     };
     request(kw0, c0, w0);
-#pragma unroll
-    for (int j = 0; j < NS - 2; j++) load_set(j, c0 + j * U);
     for (int ci = c0;;) {
 #pragma unroll
         for (int j = 0; j < NS; j++) {
