@@ -120,13 +120,10 @@ __device__ __forceinline__ void bwdx_rows_body(const Geom &g, const RowTeams &rt
 // last channel where the count is not a multiple of U (same values in, same values out), and
 // the ReLU mask of the layer below comes from one load before the loop; the number of accesses
 // in flight is then the same on every path and the waits are for exactly the set that is needed.
-#ifndef MSD_RING_SETS
-#define MSD_RING_SETS 4
-#endif
 // s_waitcnt for the scalar (and LDS) counter alone: lgkmcnt(0), the vector-memory and export
 // counters at their maxima
 constexpr int kWaitScalarLoads = 0xC07F;
-constexpr int kRingSets = MSD_RING_SETS;                     // kAhead = kRingSets - 2 steps
+constexpr int kRingSets = 4;                     // kAhead = kRingSets - 2 steps (three to seven sets time alike)
 
 template <int NDIM, int V, int U>
 __device__ __forceinline__ void bwdx_pair_body(const Geom &g, const RowTeams &rt, int cch, int remap,
