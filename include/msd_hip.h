@@ -84,7 +84,9 @@ int msd_set_kernel_path(int path);
  * input and 4 output channels), "block.split3d" (the backward pass of a 3D block of one-channel
  * layers; 1: a chain of backward_x launches on the caller's stream and the weight gradients, two
  * layers per pass, on a second stream that is forked from and joined to the caller's inside the
- * call; 2: the same launches on the caller's stream alone; 0: one fused launch per layer).
+ * call; 2: the same launches on the caller's stream alone; 0: one fused launch per layer),
+ * "block.chainpair" (0/1: that chain takes two layers per read-modify-write pass over
+ * grad_input where it can; 0: one launch per layer).
  * Unknown keys return MSD_ERR_INVALID.
  */
 int msd_set_tuning(const char *key, int value);

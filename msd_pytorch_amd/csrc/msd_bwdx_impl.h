@@ -376,8 +376,9 @@ int pair_vec(const Geom &g, const View<const float> &gy, const View<float> &gx)
 {
     if (g.Wd != 2 || gx.sx != 1 || gy.sx != 1) return 0;
     const int vmax = knob(NDIM == 3 ? kKnobBwdxVec3d : kKnobBwdxVec2d, NDIM == 3 ? 1 : 4);
+    // (two voxels per lane at most: four would hold 216 gathered values per lane)
     for (int pass = 0; pass < 2; pass++)
-        for (int v = 4; v >= 1; v /= 2) {
+        for (int v = 2; v >= 1; v /= 2) {
             if (pass == 0 && v > vmax) continue;
             if (!rows_aligned(gx, g.W, v) || !rows_aligned(gy, g.W, v) || !fits<NDIM>(g, v, 2)) continue;
             RowTeams rt;
@@ -406,7 +407,6 @@ hipError_t pair_nd(const Geom &g, const View<const float> &gy, const float *k, c
     g2.dil = group->dil[0];
     const UpperDilations up{{group->dil[1], 0}};
     const int v = pair_vec<NDIM>(g2, gy, gx);
-    if (v == 4) return pair_unroll<NDIM, 4>(g2, gy, k, gx, pm, s, group->k_up[0], up);
     if (v == 2) return pair_unroll<NDIM, 2>(g2, gy, k, gx, pm, s, group->k_up[0], up);
     if (v == 1) return pair_unroll<NDIM, 1>(g2, gy, k, gx, pm, s, group->k_up[0], up);
     return hipErrorInvalidConfiguration;
