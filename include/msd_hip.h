@@ -86,7 +86,9 @@ int msd_set_kernel_path(int path);
  * layers per pass, on a second stream that is forked from and joined to the caller's inside the
  * call; 2: the same launches on the caller's stream alone; 0: one fused launch per layer),
  * "block.chainpair" (0/1: that chain takes two layers per read-modify-write pass over
- * grad_input where it can; 0: one launch per layer).
+ * grad_input where it can; 0: one launch per layer), "bwdk.fused3d" (0/1: the weight gradient of
+ * a 3D layer of one or two output channels runs on the weight-gradient-only form of the fused
+ * backward kernel where that takes the shape; 0: on the separate weight-gradient kernels).
  * Unknown keys return MSD_ERR_INVALID.
  */
 int msd_set_tuning(const char *key, int value);

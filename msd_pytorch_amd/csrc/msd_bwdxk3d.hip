@@ -31,4 +31,15 @@ hipError_t fast_backward_k_pair_3d(const Geom &g, const View<const float> &gy, c
     return bwdxk::k_pair_3d(g, gy, x, gk, gb, ws, s, defer, group);
 }
 
+bool fast_backward_k_only_supported_3d(const Geom &g, const View<const float> &gy, const View<const float> &x)
+{
+    return bwdxk::k_only_supported_3d(g, gy, x);
+}
+
+hipError_t fast_backward_k_only_3d(const Geom &g, const View<const float> &gy, const View<const float> &x, float *gk,
+                                   float *gb, float *ws, hipStream_t s)
+{
+    return bwdxk::k_only_3d(g, gy, x, gk, gb, ws, s);
+}
+
 }  // namespace msd

@@ -1103,5 +1103,34 @@ inline hipError_t k_pair_3d(const Geom &g, const View<const float> &gy, const Vi
     return launch<3, 1, 4, 2, false, false, true>(g, gy, x, nullptr, none, pm, gk, gb, ws, s, defer, group);
 }
 
+// Weight and bias gradients of one 3D layer of one or two output channels (one dilation) from
+// its masked output gradient: the same instances without a group, and those of one output
+// channel.
+inline bool k_only_supported_3d(const Geom &g, const View<const float> &gy, const View<const float> &x)
+{
+    if (g.ndim != 3 || g.Wd < 1 || g.Wd > 2 || x.sx != 1 || gy.sx != 1) return false;
+    if (!small_strides(g, gy) || !small_strides(g, x) || !x_offsets_fit(g, x, false)) return false;
+    const View<float> none{const_cast<float *>(gy.p), gy.sb, gy.sc, gy.sz, gy.sy, gy.sx};   // (grad_input is not touched)
+    return fits<3>(g, 1, gy, x, none, false);
+}
+
+template <int WOUT>
+inline hipError_t k_only_3d_w(const Geom &g, const View<const float> &gy, const View<const float> &x, float *gk,
+                              float *gb, float *ws, hipStream_t s)
+{
+    const View<float> none{nullptr, 0, 0, 0, 0, 1};
+    const PostMask pm{g.C, {nullptr, 0, 0, 0, 0, 0}};
+    const int need = (g.C + kChanBlock - 1) / kChanBlock;
+    if (need <= 1) return launch<3, 1, 1, WOUT, false, false, true>(g, gy, x, nullptr, none, pm, gk, gb, ws, s, nullptr, nullptr);
+    if (need <= 2) return launch<3, 1, 2, WOUT, false, false, true>(g, gy, x, nullptr, none, pm, gk, gb, ws, s, nullptr, nullptr);
+    return launch<3, 1, 4, WOUT, false, false, true>(g, gy, x, nullptr, none, pm, gk, gb, ws, s, nullptr, nullptr);
+}
+
+inline hipError_t k_only_3d(const Geom &g, const View<const float> &gy, const View<const float> &x, float *gk, float *gb,
+                            float *ws, hipStream_t s)
+{
+    return g.Wd == 1 ? k_only_3d_w<1>(g, gy, x, gk, gb, ws, s) : k_only_3d_w<2>(g, gy, x, gk, gb, ws, s);
+}
+
 }  // namespace bwdxk
 }  // namespace msd

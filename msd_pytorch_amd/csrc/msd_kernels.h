@@ -61,7 +61,7 @@ enum Knob {
     kKnobXcdRemap, kKnobBwdkVec2d, kKnobBwdkVec3d, kKnobBwdkBlocks,
     kKnobFwdVec2d, kKnobFwdVec3d, kKnobFwdSplit, kKnobFwdRows2d, kKnobBwdkRows, kKnobBlockFuse,
     kKnobBlockDefer, kKnobBwdkInterleave, kKnobBlockSnake, kKnobFwdClass3d, kKnobFwdLattice3d,
-    kKnobBlockPair, kKnobBlockTriple, kKnobFinalTiled, kKnobBlockSplit3d, kKnobBlockChainPair,
+    kKnobBlockPair, kKnobBlockTriple, kKnobFinalTiled, kKnobBlockSplit3d, kKnobBlockChainPair, kKnobBwdkFused3d,
     kKnobCount
 };
 int knob(Knob k, int dflt);
@@ -194,6 +194,13 @@ hipError_t fast_backward_xkb_3d(const Geom &g, const View<const float> &gy, cons
 bool fast_backward_k_pair_supported_3d(const Geom &g, const View<const float> &gy, const View<const float> &x);
 hipError_t fast_backward_k_pair_3d(const Geom &g, const View<const float> &gy, const View<const float> &x, float *gk,
                                    float *gb, float *ws, hipStream_t s, ReduceJob *defer, const LayerGroup *group);
+// Weight and bias gradients of one 3D layer of one or two output channels from its masked
+// output gradient, by the same kernel (no grad_input is touched; gk must not be null, gb may
+// be); partial sums behind the first backward_k_mask_floats(g) floats of ws, as for
+// fast_backward_kb.
+bool fast_backward_k_only_supported_3d(const Geom &g, const View<const float> &gy, const View<const float> &x);
+hipError_t fast_backward_k_only_3d(const Geom &g, const View<const float> &gy, const View<const float> &x, float *gk,
+                                   float *gb, float *ws, hipStream_t s);
 // grad_input of two 3D layers of a dense block (one output channel each, own dilations) in one
 // read-modify-write pass over the g.C input channels they share: output channel 0 is the lower
 // layer (k, group->dil[0]), output channel 1 the upper one (group->k_up[0], group->dil[1]); gy

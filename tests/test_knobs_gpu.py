@@ -62,11 +62,14 @@ FORWARD_3D += [({"fwd.lattice3d": 44, "fwd.split": k}, VOL_E) for k in (1, 4)]
 SPLIT = [({"fwd.split": k}, s) for k in (1, 2, 4) for s in (IMG_A, IMG_C, VOL_A, VOL_C)]
 ORDER = [({"xcd_remap": r}, s) for r in (0, 1) for s in (IMG_B, IMG_D, VOL_A, VOL_D)]
 BACKWARD_K = [({"bwdk.vec2d": v}, s) for v in (1, 2, 4) for s in (IMG_A, IMG_B, IMG_C)]
-BACKWARD_K += [({"bwdk.vec3d": v}, s) for v in (1, 2) for s in (VOL_A, VOL_B)]
-BACKWARD_K += [({"bwdk.rows": r}, s) for r in (0, 1) for s in (IMG_A, IMG_B, VOL_A)]
+# ("bwdk.fused3d": 0 keeps a 3D layer of one or two output channels on the kernels that these
+# parameters shape; by default it goes through the weight-gradient-only form of the fused kernel)
+BACKWARD_K += [({"bwdk.vec3d": v, "bwdk.fused3d": 0}, s) for v in (1, 2) for s in (VOL_A, VOL_B)]
+BACKWARD_K += [({"bwdk.fused3d": f}, s) for f in (0, 1) for s in (VOL_A, VOL_B, VOL_C, VOL_D, VOL_E)]
+BACKWARD_K += [({"bwdk.rows": r, "bwdk.fused3d": 0}, s) for r in (0, 1) for s in (IMG_A, IMG_B, VOL_A)]
 BACKWARD_K += [({"bwdk.rows": 0, "bwdk.vec2d": v}, IMG_B) for v in (2, 4)]
-BACKWARD_K += [({"bwdk.interleave": i}, s) for i in (0, 1) for s in (IMG_D, VOL_D)]
-BACKWARD_K += [({"bwdk.blocks": n}, s) for n in (8, 40) for s in (IMG_D, VOL_A)]
+BACKWARD_K += [({"bwdk.interleave": i, "bwdk.fused3d": f}, s) for i in (0, 1) for f in (0, 1) for s in (IMG_D, VOL_D)]
+BACKWARD_K += [({"bwdk.blocks": n, "bwdk.fused3d": f}, s) for n in (8, 40) for f in (0, 1) for s in (IMG_D, VOL_A)]
 BACKWARD_X = [({"bwdx.vec2d": v, "bwdx.unroll2d": u}, s) for v in (1, 2, 4) for u in (2, 4) for s in (IMG_A, IMG_C)]
 BACKWARD_X += [({"bwdx.vec3d": v, "bwdx.unroll3d": u}, s) for v in (1, 2, 4) for u in (2, 4) for s in (VOL_B, VOL_C)]
 BACKWARD_X += [({"bwdx.min_blocks": n}, s) for n in (1, 4096) for s in (IMG_B, VOL_B)]
@@ -93,19 +96,19 @@ INSTANCES = [
     ({"bwdk.rows": 0, "bwdk.vec2d": 2}, (1, 70, 1, (9, 256), 2)),
     ({"bwdk.rows": 0, "bwdk.vec2d": 2}, (1, 3, 1, (9, 256), 2)),
     ({"bwdk.rows": 0, "bwdk.vec2d": 4}, (1, 40, 1, (9, 256), 2)),
-    ({"bwdk.rows": 0, "bwdk.vec3d": 2}, (1, 40, 1, (5, 6, 128), 2)),
-    ({"bwdk.rows": 0, "bwdk.vec3d": 4}, (1, 3, 1, (5, 6, 128), 2)),
-    ({"bwdk.rows": 0, "bwdk.vec3d": 4}, (1, 20, 1, (5, 6, 128), 2)),
-    ({"bwdk.rows": 0, "bwdk.vec3d": 4}, (1, 40, 1, (5, 6, 128), 2)),
-    ({"bwdk.rows": 0, "bwdk.vec3d": 4}, (1, 70, 1, (5, 6, 128), 2)),
+    ({"bwdk.rows": 0, "bwdk.vec3d": 2, "bwdk.fused3d": 0}, (1, 40, 1, (5, 6, 128), 2)),
+    ({"bwdk.rows": 0, "bwdk.vec3d": 4, "bwdk.fused3d": 0}, (1, 3, 1, (5, 6, 128), 2)),
+    ({"bwdk.rows": 0, "bwdk.vec3d": 4, "bwdk.fused3d": 0}, (1, 20, 1, (5, 6, 128), 2)),
+    ({"bwdk.rows": 0, "bwdk.vec3d": 4, "bwdk.fused3d": 0}, (1, 40, 1, (5, 6, 128), 2)),
+    ({"bwdk.rows": 0, "bwdk.vec3d": 4, "bwdk.fused3d": 0}, (1, 70, 1, (5, 6, 128), 2)),
     ({"bwdk.vec2d": 1}, (1, 40, 1, (9, 128), 2)),
     ({"bwdk.vec2d": 1}, (1, 70, 1, (9, 128), 2)),   # one voxel per lane, one output channel, > 64 channels
     ({"bwdk.vec2d": 2}, (1, 70, 1, (9, 128), 2)),
     ({"bwdk.vec2d": 4}, (1, 70, 1, (9, 256), 2)),
-    ({"bwdk.vec3d": 1}, (1, 20, 1, (5, 6, 64), 2)),
-    ({"bwdk.vec3d": 1}, (1, 40, 1, (5, 6, 64), 2)),
-    ({"bwdk.vec3d": 2}, (1, 40, 1, (5, 6, 128), 2)),
-    ({"bwdk.vec3d": 2}, (1, 70, 1, (5, 6, 128), 2)),
+    ({"bwdk.vec3d": 1, "bwdk.fused3d": 0}, (1, 20, 1, (5, 6, 64), 2)),
+    ({"bwdk.vec3d": 1, "bwdk.fused3d": 0}, (1, 40, 1, (5, 6, 64), 2)),
+    ({"bwdk.vec3d": 2, "bwdk.fused3d": 0}, (1, 40, 1, (5, 6, 128), 2)),
+    ({"bwdk.vec3d": 2, "bwdk.fused3d": 0}, (1, 70, 1, (5, 6, 128), 2)),
     ({"bwdx.vec2d": 4, "bwdx.unroll2d": 4}, (1, 5, 1, (4, 2048), 3)),     # rows of 512 lanes
     ({"bwdx.vec2d": 4, "bwdx.unroll2d": 4}, (1, 5, 2, (4, 2048), 3)),
     ({"bwdx.vec3d": 4, "bwdx.unroll3d": 2}, (1, 5, 1, (3, 4, 2048), 3)),
@@ -170,7 +173,7 @@ INSTANCES = [
     ({}, (2, 20, 1, (4, 3, 384), 2)),
     ({}, (1, 40, 1, (3, 5, 512), 1)),
     ({}, (1, 70, 1, (2, 4, 512), 2)),
-    ({"bwdk.vec3d": 2}, (1, 20, 1, (5, 6, 128), 2)),
+    ({"bwdk.vec3d": 2, "bwdk.fused3d": 0}, (1, 20, 1, (5, 6, 128), 2)),
     ({}, (1, 40, 1, (4, 5, 130), 2)),                # 3D rows that are not whole groups of four voxels, 33-64 channels
 ]
 
@@ -179,6 +182,10 @@ def _id(case):
     settings, s = case
     knobs = ",".join("%s=%d" % kv for kv in settings.items())
     return "%s-B%d-C%d-w%d-%s-d%d" % (knobs, s[0], s[1], s[2], "x".join(map(str, s[3])), s[4])
+
+
+# the 3D entries without a setting of their own once more on the separate weight-gradient kernels
+INSTANCES += [({"bwdk.fused3d": 0}, shape) for settings, shape in INSTANCES if not settings and len(shape[3]) == 3]
 
 
 @pytest.mark.parametrize("case", FORWARD_2D + FORWARD_3D + SPLIT + ORDER + BACKWARD_K + BACKWARD_X + INSTANCES,
