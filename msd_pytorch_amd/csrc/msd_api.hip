@@ -1005,13 +1005,11 @@ int block_backward_split3d(const char *fn, const BlockArgs &a, int64_t c_in, con
                            bool *done)
 {
     *done = false;
-    // By default for volumes of up to 4 M voxels: the two streams gain what the launches' ramps
-    // and tails leave idle (about 15 to 30 microseconds per launch), the separate kernels lose a
-    // share of the fused pass's time that grows with the volume (128^3, depth 50: 7.7 against
-    // 8.2 ms; 256^3, depth 30: 28.9 against 25.0 ms).
-    int64_t voxels = a.batch;
-    for (int d = 0; d < a.ndim; d++) voxels *= a.spatial[d];
-    const int mode = msd::knob(msd::kKnobBlockSplit3d, voxels <= ((int64_t)1 << 22) ? 1 : 0);
+    // By default wherever the kernels take the shapes: the two streams gain what the launches'
+    // ramps and tails leave idle (about 15 to 30 microseconds per launch) and the chain moves half
+    // the bytes of grad_input (128^3, depth 50: 6.8 against 8.2 ms for the backward pass; 256^3,
+    // depth 30: 35.0 against 35.9 ms per step; 160 x 160 x 256, depth 50: 30.7 against 34.0 ms).
+    const int mode = msd::knob(msd::kKnobBlockSplit3d, 1);
     if (mode == 0 || a.dtype != MSD_F32 || a.ndim != 3 || g_kernel_path != 0 || !grad_bias || a.depth < 2 ||
         !msd::knob(msd::kKnobBlockFuse, 1))
         return MSD_OK;
