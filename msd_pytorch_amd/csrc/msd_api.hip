@@ -890,6 +890,7 @@ int block_group_fused(const char *fn, const BlockArgs &a, int i, int n, int64_t 
         int dmax = 0;
         st.group.n = j;
         st.group.lowest_channels = 0;
+        st.group.max_workgroups = 0;
         for (int q = 0; q < j; q++) {
             st.group.dil[q] = (int)a.dilations[bottom + q];
             dmax = st.group.dil[q] > dmax ? st.group.dil[q] : dmax;
@@ -964,6 +965,7 @@ struct SideStream {
     size_t next = 0;
 };
 constexpr int kSideEvents = 32;
+constexpr int kSideWorkgroups = 384;          // of the weight-gradient pass while the chain runs beside it
 std::mutex g_side_mutex;
 SideStream g_side[64];
 
@@ -1071,6 +1073,7 @@ int block_backward_split3d(const char *fn, const BlockArgs &a, int64_t c_in, con
             st.group.k_up[1] = nullptr;
             st.group.gk_up[0] = st.group.gk_up[1] = nullptr;
             st.group.lowest_channels = 0;
+            st.group.max_workgroups = 0;
             st.gx = gx;
             st.k = (const float *)weights[i];
             st.pm = i > 0 ? msd::PostMask{(int)(first - 1), x} : msd::PostMask{(int)first, {nullptr, 0, 0, 0, 0, 0}};
@@ -1089,6 +1092,7 @@ int block_backward_split3d(const char *fn, const BlockArgs &a, int64_t c_in, con
             p.group.gk_up[0] = (float *)grad_weights[i + 1];
             p.group.gk_up[1] = nullptr;
             p.group.lowest_channels = (int)first;
+            p.group.max_workgroups = 0;
             p.gy = gy;                            // channels first (layer i) and first + 1 (layer i + 1)
             if (!msd::fast_backward_k_pair_supported_3d(p.g, p.gy, x)) return MSD_OK;
             MSD_TRY(check_workspace(fn, p.g, sizeof(float), workspace, workspace_bytes));
@@ -1125,6 +1129,11 @@ int block_backward_split3d(const char *fn, const BlockArgs &a, int64_t c_in, con
             MSD_TRY(pending->next(fn, region, &job));
             ProfileScope scope(2, ks);
             p.g.reverse = msd::knob(msd::kKnobBlockSnake, 1) && (i & 2);
+            // beside the chain, three quarters of the workgroups that would be resident alone:
+            // the chain's workgroups find room on every compute unit (128^3, depth 50: 10.0
+            // against 10.2 ms per step; 256^3: 33.9 against 34.9; alone on the chip the full
+            // number is faster, 10.8 against 11.8 ms)
+            p.group.max_workgroups = side ? kSideWorkgroups : 0;
             const hipError_t e = msd::fast_backward_k_pair_3d(p.g, p.gy, x, (float *)grad_weights[i],
                                                               (float *)grad_bias + i, (float *)workspace, ks, job,
                                                               &p.group);

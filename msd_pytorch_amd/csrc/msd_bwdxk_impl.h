@@ -875,7 +875,10 @@ hipError_t launch(const Geom &g, const View<const float> &gy, const View<const f
     a.remap = knob(kKnobXcdRemap, 1);
     // as many workgroups as are resident at once (256 CUs): the grid then runs as one round
     const int64_t max_wgs = std::min<int64_t>(
-        std::max(8, knob(kKnobBwdkBlocks, 256 * resident_per_cu<NDIM, V, NCB, WOUT, LONG>())), kMaxPartialRows);
+        std::max(8, knob(kKnobBwdkBlocks, group && group->max_workgroups > 0
+                                              ? group->max_workgroups
+                                              : 256 * resident_per_cu<NDIM, V, NCB, WOUT, LONG>())),
+        kMaxPartialRows);
     a.tiles_per_wg = (int)((total + max_wgs - 1) / max_wgs);
     const int64_t wgs = (total + a.tiles_per_wg - 1) / a.tiles_per_wg;
     const int rows = a.remap ? xcd_grid((int)wgs) : (int)wgs;   // padding workgroups write zero rows

@@ -166,6 +166,7 @@ struct LayerGroup {
     const float *k_up[kMaxLayerGroup - 1];
     float *gk_up[kMaxLayerGroup - 1];
     int lowest_channels;   // > 0: the lowest layer has only this many of the pass's input channels
+    int max_workgroups;    // > 0: workgroups of the launch (a pass that shares the chip with another stream's)
 };
 constexpr int kReduceBatch = 16;
 // One launch for up to kReduceBatch pending reductions; every column is added in the same
