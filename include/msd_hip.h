@@ -88,7 +88,9 @@ int msd_set_kernel_path(int path);
  * "block.chainpair" (0/1: that chain takes two layers per read-modify-write pass over
  * grad_input where it can; 0: one launch per layer), "bwdk.fused3d" (0/1: the weight gradient of
  * a 3D layer of one or two output channels runs on the weight-gradient-only form of the fused
- * backward kernel where that takes the shape; 0: on the separate weight-gradient kernels).
+ * backward kernel where that takes the shape; 0: on the separate weight-gradient kernels),
+ * "bwdx.lean1" (0/1: a 3D backward_x over one input and one output channel runs on a kernel
+ * of its own; 0: on the general one).
  * Unknown keys return MSD_ERR_INVALID.
  */
 int msd_set_tuning(const char *key, int value);

@@ -50,7 +50,7 @@ SWEEP_GRID = {
     },
     "backward_kb": {
         2: {"bwdk.vec2d": (1, 2, 4), "bwdk.rows": (0, 1), "bwdk.blocks": (256, 512, 1024)},
-        3: {"bwdk.vec3d": (1, 2), "bwdk.rows": (0, 1), "bwdk.blocks": (256, 512, 1024)},
+        3: {"bwdk.fused3d": (0, 1), "bwdk.vec3d": (1, 2), "bwdk.rows": (0, 1), "bwdk.blocks": (256, 512, 1024)},
     },
     "backward_xkb": {
         2: {"bwdk.vec2d": (1, 2, 4), "bwdk.blocks": (256, 512, 768, 1024), "bwdk.interleave": (0, 1)},

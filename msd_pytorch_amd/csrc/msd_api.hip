@@ -17,9 +17,9 @@ const char *const kKnobNames[kKnobCount] = {
     "xcd_remap", "bwdk.vec2d", "bwdk.vec3d", "bwdk.blocks",
     "fwd.vec2d", "fwd.vec3d", "fwd.split", "fwd.rows2d", "bwdk.rows", "block.fuse",
     "block.defer", "bwdk.interleave", "block.snake", "fwd.class3d", "fwd.lattice3d",
-    "block.pair", "block.triple", "final.tiled", "block.split3d", "block.chainpair", "bwdk.fused3d",
+    "block.pair", "block.triple", "final.tiled", "block.split3d", "block.chainpair", "bwdk.fused3d", "bwdx.lean1",
 };
-static_assert(kKnobBwdkFused3d + 1 == kKnobCount, "one name per knob, in the order of the enum");
+static_assert(kKnobBwdxLean1 + 1 == kKnobCount, "one name per knob, in the order of the enum");
 int g_knobs[kKnobCount];
 // every knob starts at "library default"
 const bool g_knobs_ready = [] {

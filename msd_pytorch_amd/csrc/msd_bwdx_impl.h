@@ -248,6 +248,95 @@ __device__ __forceinline__ void bwdx_pair_body(const Geom &g, const RowTeams &rt
     }
 }
 
+constexpr size_t kMaxLdsOneChannel = 64 * 1024;
+
+// One input channel, one output channel (the step of the dense block's chain in which the upper
+// layer of a pair finishes the channel the lower layer wrote): there is no channel loop to keep
+// the gathered taps for, so they are multiplied as they are read from the staged rows and a
+// lane can own four voxels at 80 registers: a quarter of the workgroups (128^3: 20 against 24
+// us with the general kernel; what remains is one launch and one chain of round trips: gather,
+// LDS, store; one, two or four voxels per lane time alike).
+template <int NDIM, int V>
+__global__ __launch_bounds__(256, 6) void bwdx_one_channel(Geom g, RowTeams rt, int remap, View<const float> gy,
+                                                           const float *__restrict__ k, View<float> gx, PostMask pm)
+{
+    extern __shared__ float lds[];
+    constexpr int NPQ = RowTaps<NDIM>::NPQ;
+    const int team = threadIdx.x / rt.lpr, lane = threadIdx.x % rt.lpr;
+    const int lb = block_for_xcd(blockIdx.x, gridDim.x, remap);
+    if (lb * rt.rpw >= rt.nrows) return;   // padding block (whole workgroup)
+    const int row = lb * rt.rpw + team;
+    const int x0 = lane * V;
+    const bool act = row < rt.nrows && x0 < g.W;
+    const int rr = min(row, rt.nrows - 1);
+    const int y = rr % g.H, z = rr / g.H;
+    const int b = blockIdx.y;
+    // the channel's own values and its activation are asked for before the gather
+    const int64_t at = (int64_t)b * gx.sb + (int64_t)z * gx.sz + (int64_t)y * gx.sy + min(x0, g.W - V);
+    float cur[V], below[V];
+    load_vec<V>(gx.p + at, cur);
+    const bool masked = pm.from < 1;
+    load_vec<V>(masked ? pm.act.p + (int64_t)b * pm.act.sb + (int64_t)z * pm.act.sz + (int64_t)y * pm.act.sy +
+                             min(x0, g.W - V)
+                       : gx.p + at,
+                below);
+    float *S = lds + (size_t)team * NPQ * V * rt.lpr;
+    float own[1][NPQ][V];
+    stage_source_rows<NDIM, false, 1, V>(g, rt, gy, gy, b, z, y, lane, act, S, own);
+    if (!act) return;
+#pragma unroll
+    for (int i = 0; i < V; i++) {
+        const SideTaps<V> side(x0 + i, g.W, g.dil, rt.lpr);
+        float s = 0.f;
+#pragma unroll
+        for (int pq = 0; pq < NPQ; pq++) {
+            float t0, t2;
+            side.read(S + (size_t)pq * V * rt.lpr, t0, t2);
+            s += k[pq * 3 + 0] * t0;
+            s += k[pq * 3 + 1] * own[0][pq][i];
+            s += k[pq * 3 + 2] * t2;
+        }
+        cur[i] += s;
+        cur[i] = masked && !(0.f < below[i]) ? 0.f : cur[i];
+    }
+    store_vec<V>(gx.p + at, cur);
+}
+
+template <int NDIM>
+int one_channel_vec(const Geom &g, const View<const float> &gy, const View<float> &gx, const PostMask &pm)
+{
+    if (g.C != 1 || g.Wd != 1 || gx.sx != 1 || gy.sx != 1 || (pm.from < 1 && pm.act.sx != 1)) return 0;
+    for (int v = 4; v >= 1; v /= 2) {
+        if (!rows_aligned(gx, g.W, v) || !rows_aligned(gy, g.W, v) || (pm.from < 1 && !rows_aligned(pm.act, g.W, v)))
+            continue;
+        RowTeams rt;
+        if (!make_row_teams(g, v, &rt) || rt.lpr * rt.rpw > 256) continue;
+        if (staged_floats<NDIM>(rt, 1) * rt.rpw * sizeof(float) <= kMaxLdsOneChannel) return v;
+    }
+    return 0;
+}
+
+template <int NDIM>
+hipError_t one_channel_nd(const Geom &g, const View<const float> &gy, const float *k, const View<float> &gx,
+                          const PostMask &pm, hipStream_t s)
+{
+    const int v = one_channel_vec<NDIM>(g, gy, gx, pm);
+    if (v == 0) return hipErrorInvalidConfiguration;
+    RowTeams rt;
+    make_row_teams(g, v, &rt);
+    const int nb = (rt.nrows + rt.rpw - 1) / rt.rpw;
+    const size_t lds = staged_floats<NDIM>(rt, 1) * rt.rpw * sizeof(float);
+    const int remap = knob(kKnobXcdRemap, 1);
+    const dim3 grid(remap ? xcd_grid(nb) : nb, g.B, 1), block(rt.lpr * rt.rpw);
+    if (v == 4)
+        hipLaunchKernelGGL((bwdx_one_channel<NDIM, 4>), grid, block, lds, s, g, rt, remap, gy, k, gx, pm);
+    else if (v == 2)
+        hipLaunchKernelGGL((bwdx_one_channel<NDIM, 2>), grid, block, lds, s, g, rt, remap, gy, k, gx, pm);
+    else
+        hipLaunchKernelGGL((bwdx_one_channel<NDIM, 1>), grid, block, lds, s, g, rt, remap, gy, k, gx, pm);
+    return hipGetLastError();
+}
+
 constexpr size_t kMaxLds = 64 * 1024;
 
 template <int NDIM, bool RELU, int WOUT, int V, int U, int MAXT>

@@ -61,7 +61,7 @@ enum Knob {
     kKnobXcdRemap, kKnobBwdkVec2d, kKnobBwdkVec3d, kKnobBwdkBlocks,
     kKnobFwdVec2d, kKnobFwdVec3d, kKnobFwdSplit, kKnobFwdRows2d, kKnobBwdkRows, kKnobBlockFuse,
     kKnobBlockDefer, kKnobBwdkInterleave, kKnobBlockSnake, kKnobFwdClass3d, kKnobFwdLattice3d,
-    kKnobBlockPair, kKnobBlockTriple, kKnobFinalTiled, kKnobBlockSplit3d, kKnobBlockChainPair, kKnobBwdkFused3d,
+    kKnobBlockPair, kKnobBlockTriple, kKnobFinalTiled, kKnobBlockSplit3d, kKnobBlockChainPair, kKnobBwdkFused3d, kKnobBwdxLean1,
     kKnobCount
 };
 int knob(Knob k, int dflt);

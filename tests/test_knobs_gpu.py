@@ -185,6 +185,11 @@ def _id(case):
     return "%s-B%d-C%d-w%d-%s-d%d" % (knobs, s[0], s[1], s[2], "x".join(map(str, s[3])), s[4])
 
 
+# 3D, one input and one output channel: the lean backward_x kernel at four, two and one voxel
+# per lane, and the general kernel on the same shapes
+INSTANCES += [(settings, shape) for settings in ({}, {"bwdx.lean1": 0})
+              for shape in ((2, 1, 1, (5, 6, 128), 2), (1, 1, 1, (4, 5, 66), 3), (1, 1, 1, (3, 5, 33), 1),
+                            (1, 1, 1, (6, 7, 256), 6))]
 # the 3D entries without a setting of their own once more on the separate weight-gradient kernels
 INSTANCES += [({"bwdk.fused3d": 0}, shape) for settings, shape in INSTANCES if not settings and len(shape[3]) == 3]
 
