@@ -32,7 +32,7 @@ PIPE = {"forward": "fp32 VALU, non-packed (78.6 TFLOP/s of the 157.3 peak)",
 
 # kernel families (as named in the profile summaries) whose HBM traffic belongs to a class
 FAMILIES = {"forward": ("fwd_lattice",), "backward_xkb": ("bwd_rows_fused", "bwd_one_channel", "reduce_columns"),
-            "backward_kb": ("bwdk_rows", "bwdk_mfma"), "backward_x": ("relu_mask", "bwdx_rows")}
+            "backward_kb": ("bwdk_rows", "bwdk_mfma"), "backward_x": ("relu_mask", "bwdx_rows", "bwdx_one_channel")}
 # families that are the second pass of an operator call, not a call of their own
 SECOND_PASS = ("reduce_columns",)
 

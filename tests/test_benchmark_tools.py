@@ -118,3 +118,22 @@ def test_timeit_helper():
     bench("synced", lambda: None, repeat=2, sync=lambda: synced.append(1), min_time=0.0)
     assert len(synced) >= 2 * 2 + 2          # two per run, at least the calibration run and two repeats
     assert format_time(1.5e-3) == "1.5 ms" and format_time(2.5e-7) == "250 ns" and format_time(125) == "2 min 5 s"
+
+
+def test_algorithmic_bytes_of_the_paired_3d_chain():
+    # workload D, depth 50: pairs (49, 48) ... (1, 0); the upper layer over the one channel the
+    # lower one wrote (4 planes), then one read-modify-write pass over the channels below
+    import bench
+    per_layer, _, n = bench.algorithmic_work("D", False, kpairs=True, chainpairs=False)
+    paired, flops, _ = bench.algorithmic_work("D", False, kpairs=True, chainpairs=True)
+    expect = 3 * n * 4                                    # the top layer's mask pass
+    for upper in range(49, 0, -2):
+        lower = upper - 1
+        expect += 4 * n * 4 + 27 * 4
+        if lower > 0:                                     # layer 0's pass would only serve the block's input
+            channels = 1 + lower
+            expect += (2 * channels + 2) * n * 4 + 2 * channels * 27 * 4
+    assert paired["backward_x"] == expect
+    assert 0.5 < paired["backward_x"] / per_layer["backward_x"] < 0.55
+    assert paired["backward_kb"] == per_layer["backward_kb"] and paired["forward"] == per_layer["forward"]
+    assert flops["backward_x"] > 0
