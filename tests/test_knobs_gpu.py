@@ -300,6 +300,7 @@ SPLIT_BLOCKS_3D = [
     ((9, 8, 64), 15, 5, 1, [1, 4, 2]),           # 16 to 20 channels: two blocks of 16 in the upper pairs
     ((6, 6, 64), 62, 5, 1, [2, 3]),              # 63 to 67 channels: two chunks of the grid
     ((7, 5, 96), 1, 5, 1, [1, 2]),               # rows the row kernels take with half-empty waves
+    ((24, 128, 128), 42, 6, 1, [1, 10, 3, 7, 5, 2]),   # the headline volume's rows, 43 to 47 channels
 ]
 SPLIT_MODES = {"two-streams": {"block.split3d": 1}, "one-stream": {"block.split3d": 2}, "fused": {"block.split3d": 0},
                "default": {}, "chain-of-single-layers": {"block.split3d": 1, "block.chainpair": 0}}
