@@ -1104,8 +1104,12 @@ int block_backward_split3d(const char *fn, const BlockArgs &a, int64_t c_in, con
     pending->s = ks;
     auto fork = [&]() -> int {                    // what follows on the second stream waits for the chain so far
         if (!side) return MSD_OK;
-        hipEvent_t e = side->events[side->next];
-        side->next = (side->next + 1) % kSideEvents;
+        hipEvent_t e;
+        {
+            std::lock_guard<std::mutex> lock(g_side_mutex);   // (calls from several host threads take turns)
+            e = side->events[side->next];
+            side->next = (side->next + 1) % kSideEvents;
+        }
         hipError_t err = hipEventRecord(e, main);
         if (err == hipSuccess) err = hipStreamWaitEvent(side->s, e, 0);
         return err == hipSuccess ? MSD_OK : hip_fail(fn, err);
